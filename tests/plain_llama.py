@@ -1,0 +1,261 @@
+"""A plain, slow Llama: whole sequences, no cache, 32-bit, one function per part.
+
+Written from the formulas of the reference's ``tokasaurus/model/llama.py`` and
+``tokasaurus/model/attention_utils.py`` (cited per function as file:line).  It
+shares no code with ``tokasaurus_amd``: it reads a model folder with the
+safetensors library directly, works on ``config.json`` as a plain dict and uses
+only elementary torch operations, so a mistake in the engine cannot hide in a
+shared helper.
+
+Where the reference delegates a formula to an installed package (the rotary
+table generator and rotation, the attention scale and mask, the sampler), the
+mathematical definition is used and pinned by invariants in
+``tests/test_plain_llama.py``.
+"""
+
+from __future__ import annotations
+
+import json
+import math
+from pathlib import Path
+
+import torch
+from safetensors import safe_open
+
+
+# --------------------------------------------------------------------------
+# parts
+# --------------------------------------------------------------------------
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """llama.py:44-53: statistics in 32-bit, cast back, then multiply by weight."""
+    dtype = x.dtype
+    xf = x.to(torch.float32)
+    variance = xf.pow(2).mean(-1, keepdim=True)
+    xf = xf * torch.rsqrt(variance + eps)
+    return weight * xf.to(dtype)
+
+
+def rope_inverse_frequencies(
+    head_dim: int, theta: float, scaling: dict | None
+) -> torch.Tensor:
+    """The table generator behind llama.py:559-570 (delegated there).
+
+    inv_freq_j = theta^(-2j/d); with rope_type "llama3" every frequency is
+    remapped by its wavelength: short waves stay, long waves are divided by
+    ``factor``, the band between is blended linearly in orig/wavelength.
+    """
+    j = torch.arange(0, head_dim, 2, dtype=torch.int64).to(torch.float32)
+    inv_freq = 1.0 / (theta ** (j / head_dim))
+    if scaling is None:
+        return inv_freq
+    kind = scaling.get("rope_type", scaling.get("type"))
+    if kind == "default":
+        return inv_freq
+    if kind == "linear":
+        return inv_freq / scaling["factor"]
+    if kind != "llama3":
+        raise ValueError(f"plain implementation knows no rope scaling {kind!r}")
+    factor = scaling["factor"]
+    low = scaling["low_freq_factor"]
+    high = scaling["high_freq_factor"]
+    orig = scaling["original_max_position_embeddings"]
+    low_freq_wavelen = orig / low
+    high_freq_wavelen = orig / high
+    wavelen = 2 * math.pi / inv_freq
+    scaled = torch.where(wavelen > low_freq_wavelen, inv_freq / factor, inv_freq)
+    smooth = (orig / wavelen - low) / (high - low)
+    blended = (1 - smooth) * inv_freq / factor + smooth * inv_freq
+    is_medium = (wavelen >= high_freq_wavelen) & (wavelen <= low_freq_wavelen)
+    return torch.where(is_medium, blended, scaled)
+
+
+def rope_tables(
+    positions: torch.Tensor, inv_freq: torch.Tensor
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """llama.py:563-570,576-577: cos/sin of [angle, angle], 32-bit, one row a position."""
+    angle = positions.to(torch.float32)[:, None] * inv_freq[None, :].to(torch.float32)
+    full = torch.cat([angle, angle], dim=-1)
+    return full.cos(), full.sin()
+
+
+def rotate_half(x: torch.Tensor) -> torch.Tensor:
+    half = x.shape[-1] // 2
+    return torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """llama.py:243-256: x [T, heads, d], cos/sin [T, d] broadcast over heads.
+
+    Lane j pairs with lane j + d/2 (the half-split convention of the checkpoint
+    format); the rotation is computed in 32-bit and rounded back.
+    """
+    dtype = x.dtype
+    xf = x.to(torch.float32)
+    out = xf * cos[:, None, :] + rotate_half(xf) * sin[:, None, :]
+    return out.to(dtype)
+
+
+def causal_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    window: int | None = None,
+) -> torch.Tensor:
+    """attention_utils.py:108-175 on one whole sequence.
+
+    q [T, nq, d], k/v [T, nkv, d]; query head h reads kv head h // (nq/nkv);
+    scores scaled by 1/sqrt(d) (the default of the kernels called at
+    llama.py:716-764, which pass no scale); causal; softmax in 32-bit.
+    ``window`` (not used by Llama) keeps only the last ``window`` keys.
+    """
+    T, nq, d = q.shape
+    nkv = k.shape[1]
+    group = nq // nkv
+    out = torch.empty_like(q)
+    pos = torch.arange(T)
+    allowed = pos[None, :] <= pos[:, None]
+    if window is not None:
+        allowed &= pos[None, :] > pos[:, None] - window
+    for h in range(nq):
+        g = h // group
+        scores = (q[:, h, :].float() @ k[:, g, :].float().T) / math.sqrt(d)
+        scores = scores.masked_fill(~allowed, float("-inf"))
+        probs = torch.softmax(scores, dim=-1)
+        out[:, h, :] = (probs @ v[:, g, :].float()).to(q.dtype)
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """nn.Linear without bias (llama.py:130-149): weight is [out, in]."""
+    return x @ weight.T
+
+
+def attention_block(
+    x: torch.Tensor,
+    w: dict[str, torch.Tensor],
+    prefix: str,
+    cfg: dict,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    window: int | None = None,
+) -> torch.Tensor:
+    """llama.py:218-287: norm, q/k/v, rotation, attention, o_proj, residual."""
+    nq = cfg["num_attention_heads"]
+    nkv = cfg.get("num_key_value_heads", nq)
+    T = x.shape[0]
+    h = rms_norm(x, w[f"{prefix}.input_layernorm.weight"], cfg["rms_norm_eps"])
+    q = linear(h, w[f"{prefix}.self_attn.q_proj.weight"]).view(T, nq, -1)
+    k = linear(h, w[f"{prefix}.self_attn.k_proj.weight"]).view(T, nkv, -1)
+    v = linear(h, w[f"{prefix}.self_attn.v_proj.weight"]).view(T, nkv, -1)
+    q = apply_rope(q, cos, sin)
+    k = apply_rope(k, cos, sin)
+    a = causal_attention(q, k, v, window=window).reshape(T, -1)
+    return x + linear(a, w[f"{prefix}.self_attn.o_proj.weight"])
+
+
+def swiglu_block(
+    x: torch.Tensor, w: dict[str, torch.Tensor], prefix: str, cfg: dict
+) -> torch.Tensor:
+    """llama.py:319-339: norm, silu(gate) * up, down, residual."""
+    h = rms_norm(x, w[f"{prefix}.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+    up = linear(h, w[f"{prefix}.mlp.up_proj.weight"])
+    gate = linear(h, w[f"{prefix}.mlp.gate_proj.weight"])
+    prod = gate * torch.sigmoid(gate) * up
+    return x + linear(prod, w[f"{prefix}.mlp.down_proj.weight"])
+
+
+def lm_head(x: torch.Tensor, w: dict[str, torch.Tensor], cfg: dict) -> torch.Tensor:
+    """llama.py:441-467, tie handling llama.py:842-845: final norm, logits in 32-bit."""
+    h = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
+    if cfg.get("tie_word_embeddings", False):
+        head = w["model.embed_tokens.weight"]
+    else:
+        head = w["lm_head.weight"]
+    return linear(h, head).float()
+
+
+# --------------------------------------------------------------------------
+# whole model
+# --------------------------------------------------------------------------
+
+
+def load_folder(folder: str | Path) -> tuple[dict, dict[str, torch.Tensor]]:
+    """config.json as a dict and every tensor of model.safetensors in 32-bit."""
+    folder = Path(folder)
+    cfg = json.loads((folder / "config.json").read_text())
+    weights = {}
+    with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
+        for name in f.keys():
+            weights[name] = f.get_tensor(name).to(torch.float32)
+    return cfg, weights
+
+
+def forward_logits(
+    cfg: dict,
+    w: dict[str, torch.Tensor],
+    token_ids: list[int],
+    first_position: int = 0,
+    layer_order: list[int] | None = None,
+    windows: dict[int, int] | None = None,
+) -> torch.Tensor:
+    """Logits [T, vocab] of one whole sequence (llama.py:644-667, 572-582).
+
+    ``first_position`` shifts every position (used by the invariance tests);
+    ``layer_order`` runs the layers in another order or twice (default 0..L-1);
+    ``windows`` maps a layer index to a sliding window (default: none).
+    """
+    d = cfg["hidden_size"] // cfg["num_attention_heads"]  # llama.py:158-159
+    ids = torch.tensor(token_ids, dtype=torch.int64)
+    x = w["model.embed_tokens.weight"][ids]  # llama.py:514-518, no scaling
+    positions = torch.arange(first_position, first_position + len(token_ids))
+    inv_freq = rope_inverse_frequencies(
+        d, float(cfg["rope_theta"]), cfg.get("rope_scaling")
+    )
+    cos, sin = rope_tables(positions, inv_freq)
+    order = layer_order if layer_order is not None else range(cfg["num_hidden_layers"])
+    for i in order:
+        prefix = f"model.layers.{i}"
+        window = (windows or {}).get(i)
+        x = attention_block(x, w, prefix, cfg, cos, sin, window=window)
+        x = swiglu_block(x, w, prefix, cfg)
+    return lm_head(x, w, cfg)
+
+
+# --------------------------------------------------------------------------
+# sampling
+# --------------------------------------------------------------------------
+
+
+def sample(logits: torch.Tensor, temperature: float, u: float) -> tuple[int, float]:
+    """llama.py:377-406 for one row: (token, log-probability of it).
+
+    temperature 0 is greedy on the raw logits with divisor 1
+    (model/types.py:302-312); otherwise softmax(logits / T) and the smallest
+    index whose cumulative probability exceeds ``u`` (inverse CDF).
+    """
+    logits = logits.to(torch.float32)
+    divisor = temperature if temperature > 0 else 1.0
+    probs = torch.softmax(logits / divisor, dim=-1)
+    if temperature == 0:
+        token = int(torch.argmax(logits))
+    else:
+        cdf = torch.cumsum(probs.double(), dim=-1)
+        token = int(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True))
+        token = min(token, logits.numel() - 1)
+    return token, float(torch.log(probs[token]))
+
+
+def greedy_generate(
+    cfg: dict, w: dict[str, torch.Tensor], prompt: list[int], max_tokens: int
+) -> list[int]:
+    """Greedy continuation by recomputing the whole sequence every token."""
+    ids = list(prompt)
+    out = []
+    for _ in range(max_tokens):
+        logits = forward_logits(cfg, w, ids)
+        token = int(torch.argmax(logits[-1]))
+        out.append(token)
+        ids.append(token)
+    return out

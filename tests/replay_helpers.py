@@ -1,0 +1,80 @@
+"""Builds traces (lists of steps) for the replay tests and collects the logits
+they produce, keyed by (request, position), so that every way of cutting the
+same requests can be compared with the plain implementation row by row."""
+
+from __future__ import annotations
+
+import torch
+
+import plain_llama
+from tokasaurus_amd.engine.batch import StepEntry
+
+
+def plain_rows(folder, requests: dict[str, list[int]]) -> dict[str, torch.Tensor]:
+    cfg, w = plain_llama.load_folder(folder)
+    return {rid: plain_llama.forward_logits(cfg, w, toks) for rid, toks in requests.items()}
+
+
+def run_steps(runner, steps: list[dict]) -> dict[tuple[str, int], torch.Tensor]:
+    """steps: [{"entries": [(id, tokens, want)], "end": [ids]}]; returns logits by
+    (request id, absolute position)."""
+    got: dict[tuple[str, int], torch.Tensor] = {}
+    held: dict[str, int] = {}
+    for step in steps:
+        entries = [StepEntry(rid, list(toks), list(want)) for rid, toks, want in step["entries"]]
+        logits = runner.step(entries).float().cpu()
+        row = 0
+        for rid, toks, want in step["entries"]:
+            start = held.get(rid, 0)
+            for w in want:
+                got[(rid, start + w)] = logits[row]
+                row += 1
+            held[rid] = start + len(toks)
+        assert row == logits.shape[0]
+        for rid in step.get("end", []):
+            runner.release(rid)
+            held.pop(rid, None)
+        runner.manager.check()
+    return got
+
+
+def whole(rid: str, tokens: list[int]) -> list[dict]:
+    return [{"entries": [(rid, tokens, list(range(len(tokens))))], "end": [rid]}]
+
+
+def tail_one_by_one(rid: str, tokens: list[int], tail: int = 32) -> list[dict]:
+    head = len(tokens) - tail
+    steps = [{"entries": [(rid, tokens[:head], list(range(head)))]}]
+    for i in range(head, len(tokens)):
+        steps.append({"entries": [(rid, [tokens[i]], [0])]})
+    steps[-1]["end"] = [rid]
+    return steps
+
+
+def portions(rid: str, tokens: list[int], sizes: list[int]) -> list[dict]:
+    steps, at, k = [], 0, 0
+    while at < len(tokens):
+        n = min(sizes[k % len(sizes)], len(tokens) - at)
+        steps.append({"entries": [(rid, tokens[at : at + n], list(range(n)))]})
+        at += n
+        k += 1
+    steps[-1]["end"] = [rid]
+    return steps
+
+
+def compare(got, want_rows: dict[str, torch.Tensor], atol: float, rtol: float) -> float:
+    """Every collected row against the plain row; returns the largest error seen.
+    On a mismatch, names the first wrong (request, position)."""
+    worst = 0.0
+    for (rid, pos), row in sorted(got.items()):
+        ref = want_rows[rid][pos]
+        err = (row - ref).abs()
+        bound = atol + rtol * ref.abs()
+        if not bool((err <= bound).all()):
+            i = int((err - bound).argmax())
+            raise AssertionError(
+                f"request {rid} position {pos}: logit {i} is {row[i].item():.6f}, plain {ref[i].item():.6f} "
+                f"(error {err[i].item():.3e}, allowed {bound[i].item():.3e})"
+            )
+        worst = max(worst, float(err.max()))
+    return worst

@@ -1,0 +1,106 @@
+"""The tests' own small configurations and model folders.
+
+A and B differ in every size and option: head counts and grouping, sizes that are
+no power of two, number of layers, vocabulary, the norms' eps, the rotary base and
+scaling, tied or separate head, page size.  ``sharp=True`` multiplies the query and
+key projections by 10 so that attention is peaked: with the plain N(0, 0.02) weights
+scores are tiny, softmax is nearly uniform, and one missing or misplaced key among
+a hundred would disappear in the tolerance.
+"""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import torch
+from safetensors import safe_open
+from safetensors.torch import save_file
+
+from tokasaurus_amd.weights import write_random_model
+
+CONFIG_A = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "num_hidden_layers": 2,
+    "hidden_size": 64,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "intermediate_size": 192,
+    "vocab_size": 512,
+    "rope_theta": 10000.0,
+    "rope_scaling": None,
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 512,
+}
+PAGE_A = 4
+
+CONFIG_B = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "num_hidden_layers": 3,
+    "hidden_size": 96,
+    "num_attention_heads": 3,
+    "num_key_value_heads": 1,
+    "intermediate_size": 256,
+    "vocab_size": 1000,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 8.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 64,
+    },
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False,
+    "max_position_embeddings": 384,
+}
+PAGE_B = 8
+
+# a third shape for the bfloat16 MFMA kernels: head size 64, page 16, group 4
+CONFIG_C = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "num_hidden_layers": 2,
+    "hidden_size": 256,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 1,
+    "intermediate_size": 320,
+    "vocab_size": 777,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 32.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 128,
+    },
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 640,
+}
+PAGE_C = 16
+
+TINY = {"A": (CONFIG_A, PAGE_A), "B": (CONFIG_B, PAGE_B), "C": (CONFIG_C, PAGE_C)}
+
+
+def make_folder(folder: Path, config: dict, seed: int, sharp: bool = True) -> Path:
+    write_random_model(folder, config, seed)
+    if sharp:
+        path = folder / "model.safetensors"
+        tensors = {}
+        with safe_open(str(path), framework="pt") as f:
+            for name in f.keys():
+                t = f.get_tensor(name)
+                if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
+                    t = (t.float() * 10.0).to(t.dtype)
+                tensors[name] = t
+        save_file(tensors, str(path))
+    return folder
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()

@@ -1,0 +1,170 @@
+"""The cache manager: which pages and which slot each live request holds.
+
+Layers (run entries) whose caches have equal needs form a *group*: one pool of
+page ids and, per request, one block table that every layer of the group uses
+(the reference has a single such group: one table per sequence shared by all
+layers, tokasaurus/manager/types.py:46, tokasaurus/model/llama.py:675-691).
+A group whose layers read only a window of keys gives pages back as soon as the
+window has passed them; a full group gives pages back when the request ends.
+Token ``pos`` of a request lives in page ``table[pos // P]`` at offset ``pos % P``
+(tokasaurus/manager/input_building.py:138-148).
+
+This class is host-side bookkeeping only; the tensors live in ``CacheStorage``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from tokasaurus_amd.cache.pages import NoSpaceException, PagePool, SlotAllocator
+from tokasaurus_amd.parts.base import CacheNeed
+
+RELEASED = -1  # table entry of a page the window has passed
+
+
+@dataclass(frozen=True)
+class CacheGroup:
+    need: CacheNeed
+    entries: tuple[int, ...]  # run entries that own storage in this group, in run order
+
+
+def plan_groups(needs: list[CacheNeed | None], cache_of: list[int | None]) -> tuple[list[CacheGroup], list[tuple[int, int] | None]]:
+    """Group the cache-owning run entries by need.
+
+    Returns the groups and, for every run entry, ``(group, index within the
+    group's storage)`` of the cache it uses (its own, or the one it reads), or
+    None for an entry without a cache."""
+    groups: list[CacheGroup] = []
+    members: dict[CacheNeed, list[int]] = {}
+    for i, need in enumerate(needs):
+        if need is not None and cache_of[i] is None:
+            members.setdefault(need, []).append(i)
+    for need, entries in members.items():
+        groups.append(CacheGroup(need, tuple(entries)))
+    where: list[tuple[int, int] | None] = []
+    for i, need in enumerate(needs):
+        if need is None:
+            where.append(None)
+            continue
+        owner = i if cache_of[i] is None else cache_of[i]
+        owner_need = needs[owner]
+        if owner_need is None:
+            raise ValueError(f"run entry {i} reads the cache of entry {owner}, which has none")
+        if (owner_need.num_kv_heads, owner_need.head_dim) != (need.num_kv_heads, need.head_dim):
+            raise ValueError(f"run entry {i} cannot read the cache of entry {owner}: head layout differs")
+        if owner_need.window and (not need.window or need.window > owner_need.window):
+            raise ValueError(f"run entry {i} reads further back than entry {owner} keeps keys")
+        g = next(gi for gi, grp in enumerate(groups) if grp.need == owner_need)
+        where.append((g, groups[g].entries.index(owner)))
+    return groups, where
+
+
+@dataclass
+class RequestCache:
+    request_id: str
+    slot: int
+    tables: list[list[int]]  # per group: page of each logical block, RELEASED once passed
+    num_tokens: int = 0  # tokens whose keys are in the cache
+    reserved_tokens: int = 0  # tokens the tables have room for
+    first_held: list[int] = field(default_factory=list)  # per group: first block not released
+
+
+class CacheManager:
+    def __init__(self, groups: list[CacheGroup], num_pages: int | list[int], page_size: int, max_slots: int):
+        if page_size <= 0:
+            raise ValueError("page_size must be positive")
+        self.groups = groups
+        self.page_size = page_size
+        counts = num_pages if isinstance(num_pages, list) else [num_pages] * len(groups)
+        self.pools = [PagePool(n) for n in counts]
+        self.slots = SlotAllocator(max_slots)
+        self.requests: dict[str, RequestCache] = {}
+
+    # ---- arithmetic
+    def blocks_for(self, num_tokens: int) -> int:
+        return -(-num_tokens // self.page_size)
+
+    def pages_needed(self, request_id: str | None, new_len: int) -> list[int]:
+        """Pages each group must still give for the request to hold ``new_len`` tokens."""
+        have = self.requests[request_id].tables if request_id in self.requests else [[] for _ in self.groups]
+        return [max(0, self.blocks_for(new_len) - len(t)) for t in have]
+
+    def can_hold(self, request_id: str | None, new_len: int) -> bool:
+        return all(n <= pool.num_free for n, pool in zip(self.pages_needed(request_id, new_len), self.pools))
+
+    def num_free_pages(self) -> list[int]:
+        return [p.num_free for p in self.pools]
+
+    # ---- life of a request
+    def admit(self, request_id: str) -> RequestCache:
+        if request_id in self.requests:
+            raise ValueError(f"request {request_id!r} is already live")
+        slot = self.slots.allocate()
+        rc = RequestCache(request_id, slot, [[] for _ in self.groups], first_held=[0] * len(self.groups))
+        self.requests[request_id] = rc
+        return rc
+
+    def reserve(self, request_id: str, new_len: int) -> None:
+        """Make room for the request to hold ``new_len`` tokens in every group,
+        or raise NoSpaceException with nothing taken."""
+        rc = self.requests[request_id]
+        if new_len <= rc.reserved_tokens:
+            return
+        need = self.pages_needed(request_id, new_len)
+        for n, pool in zip(need, self.pools):
+            if n > pool.num_free:
+                raise NoSpaceException(
+                    f"request {request_id!r} needs {need} more pages for {new_len} tokens, "
+                    f"free: {self.num_free_pages()}"
+                )
+        for table, n, pool in zip(rc.tables, need, self.pools):
+            table.extend(pool.allocate(n))
+        rc.reserved_tokens = self.blocks_for(new_len) * self.page_size
+
+    def advance(self, request_id: str, new_len: int) -> None:
+        """The request now holds ``new_len`` tokens: pages of windowed groups
+        that no later token can read go back to their pool."""
+        rc = self.requests[request_id]
+        if new_len > rc.reserved_tokens:
+            raise ValueError(f"request {request_id!r}: {new_len} tokens but room for {rc.reserved_tokens}")
+        if new_len < rc.num_tokens:
+            raise ValueError(f"request {request_id!r} cannot shrink")
+        rc.num_tokens = new_len
+        P = self.page_size
+        for g, grp in enumerate(self.groups):
+            w = grp.need.window
+            if not w:
+                continue
+            # the next query sits at position >= new_len and reads from new_len - w + 1 on
+            first_needed = max(0, new_len - w + 1) // P
+            table = rc.tables[g]
+            gone = []
+            for b in range(rc.first_held[g], min(first_needed, len(table))):
+                if table[b] != RELEASED:
+                    gone.append(table[b])
+                    table[b] = RELEASED
+            if gone:
+                self.pools[g].free(gone)
+            rc.first_held[g] = max(rc.first_held[g], min(first_needed, len(table)))
+
+    def release(self, request_id: str) -> None:
+        """The request is over: every page and the slot go back."""
+        rc = self.requests.pop(request_id)
+        for table, pool in zip(rc.tables, self.pools):
+            pool.free([p for p in table if p != RELEASED])
+        self.slots.free(rc.slot)
+
+    # ---- invariants (the reference's sanity_checks, allocator.py:158-194, without the tree)
+    def check(self) -> None:
+        for g, pool in enumerate(self.pools):
+            pool.check()
+            owned: list[int] = []
+            for rc in self.requests.values():
+                owned.extend(p for p in rc.tables[g] if p != RELEASED)
+            assert len(owned) == len(set(owned)), f"group {g}: a page is held by two requests"
+            assert set(owned) == pool.held_pages(), f"group {g}: tables and pool disagree"
+        self.slots.check()
+        slots = [rc.slot for rc in self.requests.values()]
+        assert len(slots) == len(set(slots)), "a slot is held by two requests"
+        for rc in self.requests.values():
+            assert rc.num_tokens <= rc.reserved_tokens

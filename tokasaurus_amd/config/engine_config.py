@@ -1,0 +1,229 @@
+"""The engine's options and the ``key=value`` command-line grammar.
+
+Names, defaults and meanings follow the reference's ``ServerConfig``
+(tokasaurus/common_types.py:52-125) for every option this engine has; the
+server, multi-GPU, hydragen and early-stopping options are not present.
+The grammar is the one the reference gets from its config library
+(README.md:93-146): ``key=value``; ``T``/``F`` for booleans; a value in
+parentheses is evaluated as a Python expression (``kv_cache_num_tokens='(512*1024)'``);
+``.name`` calls the config's method ``name``.
+"""
+
+from __future__ import annotations
+
+import ast
+import json
+import operator
+from dataclasses import dataclass, fields
+from typing import Any, get_args, get_origin, get_type_hints
+
+
+class OptionError(ValueError):
+    """A command-line argument the engine cannot accept."""
+
+
+@dataclass
+class EngineConfig:
+    # --- model (tokasaurus/common_types.py:53-58)
+    model: str | None = None
+    dtype: str = "bfloat16"
+    rope_scaling: str | None = None
+
+    # --- cache and step limits (tokasaurus/common_types.py:75-85,104)
+    page_size: int = 16
+    kv_cache_num_tokens: int = 1024 * 128
+    max_tokens_per_forward: int = 8192
+    max_seqs_per_forward: int = 1024
+    max_num_tokens_per_request: int | None = None
+    prefill_round_up_multiple: int = 16
+    greedy_prefill: bool = True
+
+    # --- outputs (tokasaurus/common_types.py:64-65)
+    enable_chosen_logprobs: bool = True
+    max_topk_logprobs: int | None = None
+
+    # --- launch-overhead removal (tokasaurus/common_types.py:117-121); here HIP graphs
+    use_hipgraphs: bool = True
+    hipgraph_max_size: int = 128
+    hipgraph_step: int = 16
+
+    # --- debugging (tokasaurus/common_types.py:124-125)
+    allocator_sanity_checks: bool = False
+    bump_city_population_me: bool = False
+
+    # --- observability (tokasaurus/common_types.py:70-71)
+    log_level: str = "INFO"
+    stats_report_seconds: float = 5.0
+
+    # --- this engine's own
+    seed: int = 0
+    max_prefill_chunk: int | None = None
+
+    def kv_cache_num_blocks(self) -> int:
+        """tokasaurus/common_types.py:130-132."""
+        if self.kv_cache_num_tokens % self.page_size:
+            raise OptionError(
+                f"kv_cache_num_tokens {self.kv_cache_num_tokens} is not a multiple of "
+                f"page_size {self.page_size}"
+            )
+        return self.kv_cache_num_tokens // self.page_size
+
+    def finalize(self, max_position_embeddings: int | None = None) -> "EngineConfig":
+        """Cross-field checks and derived values (tokasaurus/common_types.py:148-174)."""
+        if self.dtype not in ("bfloat16", "float32"):
+            raise OptionError(f"dtype {self.dtype!r}: this engine runs bfloat16 or float32")
+        for name in ("page_size", "kv_cache_num_tokens", "max_tokens_per_forward", "max_seqs_per_forward"):
+            if getattr(self, name) <= 0:
+                raise OptionError(f"{name} must be positive")
+        self.kv_cache_num_blocks()
+        if self.max_num_tokens_per_request is None and max_position_embeddings is not None:
+            self.max_num_tokens_per_request = min(max_position_embeddings, self.kv_cache_num_tokens)
+        if self.rope_scaling is not None:
+            try:
+                json.loads(self.rope_scaling)
+            except json.JSONDecodeError as e:
+                raise OptionError(f"rope_scaling is not JSON: {e}") from None
+        return self
+
+    def rope_scaling_override(self) -> tuple[bool, dict | None]:
+        if self.rope_scaling is None:
+            return False, None
+        return True, json.loads(self.rope_scaling)
+
+    # method options in the reference's manner (".name" on the command line)
+    def eager(self) -> None:
+        """``.eager``: no HIP graphs."""
+        self.use_hipgraphs = False
+
+    def fp32(self) -> None:
+        """``.fp32``: the true 32-bit path."""
+        self.dtype = "float32"
+
+
+# --------------------------------------------------------------------------
+# key=value grammar
+# --------------------------------------------------------------------------
+
+_BIN = {
+    ast.Add: operator.add,
+    ast.Sub: operator.sub,
+    ast.Mult: operator.mul,
+    ast.FloorDiv: operator.floordiv,
+    ast.Div: operator.truediv,
+    ast.Pow: operator.pow,
+    ast.Mod: operator.mod,
+    ast.LShift: operator.lshift,
+}
+
+
+def _eval_expr(text: str) -> Any:
+    """Evaluate ``(expr)``: numbers, lists, tuples, None/True/False and arithmetic."""
+
+    def ev(node: ast.AST) -> Any:
+        if isinstance(node, ast.Expression):
+            return ev(node.body)
+        if isinstance(node, ast.Constant):
+            return node.value
+        if isinstance(node, ast.BinOp) and type(node.op) in _BIN:
+            return _BIN[type(node.op)](ev(node.left), ev(node.right))
+        if isinstance(node, ast.UnaryOp) and isinstance(node.op, (ast.USub, ast.UAdd)):
+            v = ev(node.operand)
+            return -v if isinstance(node.op, ast.USub) else v
+        if isinstance(node, (ast.List, ast.Tuple)):
+            return [ev(e) for e in node.elts]
+        raise OptionError(f"expression {text!r} uses something other than literals and arithmetic")
+
+    try:
+        return ev(ast.parse(text, mode="eval"))
+    except SyntaxError as e:
+        raise OptionError(f"cannot parse expression {text!r}: {e}") from None
+
+
+def _allows_none(tp: Any) -> bool:
+    return type(None) in get_args(tp)
+
+
+def _base_type(tp: Any) -> Any:
+    args = [a for a in get_args(tp) if a is not type(None)]
+    if get_origin(tp) is not None and args:
+        return args[0] if len(args) == 1 else tuple(args)
+    return tp
+
+
+def parse_value(raw: str, tp: Any, key: str) -> Any:
+    """One value of the grammar, converted to the annotated type of its field."""
+    if raw.startswith("(") and raw.endswith(")"):
+        value = _eval_expr(raw[1:-1])
+    elif raw in ("None", "none", "null") and _allows_none(tp):
+        return None
+    else:
+        value = raw
+    base = _base_type(tp)
+    origin = get_origin(base) or base
+    if value is None:
+        if _allows_none(tp):
+            return None
+        raise OptionError(f"{key} cannot be None")
+    if origin is bool:
+        if isinstance(value, bool):
+            return value
+        if value in ("T", "True", "true", "1"):
+            return True
+        if value in ("F", "False", "false", "0"):
+            return False
+        raise OptionError(f"{key}: expected T or F, got {raw!r}")
+    if origin is int:
+        if isinstance(value, bool):
+            raise OptionError(f"{key}: expected an integer, got {raw!r}")
+        if isinstance(value, float):
+            if value != int(value):
+                raise OptionError(f"{key}: expected an integer, got {raw!r}")
+            return int(value)
+        try:
+            return int(value)
+        except (TypeError, ValueError):
+            raise OptionError(f"{key}: expected an integer, got {raw!r}") from None
+    if origin is float:
+        try:
+            return float(value)
+        except (TypeError, ValueError):
+            raise OptionError(f"{key}: expected a number, got {raw!r}") from None
+    if origin is str:
+        return str(value)
+    if origin in (list, tuple):
+        if isinstance(value, str):
+            value = _eval_expr(value)
+        if not isinstance(value, list):
+            raise OptionError(f"{key}: expected a list, got {raw!r}")
+        return value
+    return value
+
+
+def apply_overrides(config: Any, args: list[str]) -> Any:
+    """Apply ``key=value`` and ``.method`` arguments to a dataclass instance
+    (the counterpart of the call at the reference's tests/test_basic.py:32-35).
+    Unknown keys and methods are errors that list what exists."""
+    hints = get_type_hints(type(config))
+    names = [f.name for f in fields(config)]
+    for arg in args:
+        if arg.startswith("."):
+            name = arg[1:]
+            method = getattr(config, name, None)
+            if name.startswith("_") or not callable(method) or name in names:
+                known = sorted(
+                    m
+                    for m in dir(type(config))
+                    if not m.startswith("_")
+                    and callable(getattr(type(config), m))
+                    and m not in ("finalize", "kv_cache_num_blocks", "rope_scaling_override")
+                )
+                raise OptionError(f"unknown method option {arg!r}; known: {known}")
+            method()
+            continue
+        if "=" not in arg:
+            raise OptionError(f"argument {arg!r} is neither key=value nor .method")
+        key, raw = arg.split("=", 1)
+        if key not in names:
+            raise OptionError(f"unknown option {key!r}; known: {sorted(names)}")
+        setattr(config, key, parse_value(raw, hints[key], key))
+    return config

@@ -1,0 +1,221 @@
+"""Typed model configurations read from a model folder's ``config.json``.
+
+The reference hands ``config.json`` to an installed package's ``AutoConfig``
+(tokasaurus/common_types.py:138-141) and reads a handful of attributes from
+it (tokasaurus/model/llama.py:123-159,559-563, tokasaurus/model/utils.py:338-340).
+Here each architecture has a small frozen dataclass that names exactly the
+keys its parts consume and refuses a file that lacks one of them.
+"""
+
+from __future__ import annotations
+
+import json
+from dataclasses import dataclass, field, fields
+from pathlib import Path
+from typing import Any, Callable
+
+
+class ConfigError(ValueError):
+    """A config.json that the architecture cannot be built from."""
+
+
+@dataclass(frozen=True)
+class RopeScaling:
+    """The ``rope_scaling`` object of config.json (consumed inside the rotary
+    table generator that tokasaurus/model/llama.py:559-561 delegates to)."""
+
+    rope_type: str
+    factor: float = 1.0
+    low_freq_factor: float | None = None
+    high_freq_factor: float | None = None
+    original_max_position_embeddings: int | None = None
+
+    @staticmethod
+    def from_dict(d: dict[str, Any] | None) -> "RopeScaling | None":
+        if d is None:
+            return None
+        kind = d.get("rope_type", d.get("type"))
+        if kind is None:
+            raise ConfigError(f"rope_scaling has no rope_type: {d}")
+        known = {f.name for f in fields(RopeScaling)} | {"type"}
+        unknown = sorted(set(d) - known)
+        if unknown:
+            raise ConfigError(f"rope_scaling has keys this engine does not know: {unknown}")
+        out = RopeScaling(
+            rope_type=str(kind),
+            factor=float(d.get("factor", 1.0)),
+            low_freq_factor=_opt(d, "low_freq_factor", float),
+            high_freq_factor=_opt(d, "high_freq_factor", float),
+            original_max_position_embeddings=_opt(d, "original_max_position_embeddings", int),
+        )
+        out.validate()
+        return out
+
+    def validate(self) -> None:
+        if self.rope_type not in ("default", "linear", "llama3"):
+            raise ConfigError(
+                f"rope_scaling.rope_type {self.rope_type!r} is not supported "
+                "(known: default, linear, llama3)"
+            )
+        if self.rope_type == "llama3":
+            missing = [
+                k
+                for k in ("low_freq_factor", "high_freq_factor", "original_max_position_embeddings")
+                if getattr(self, k) is None
+            ]
+            if missing:
+                raise ConfigError(f"rope_scaling of type llama3 lacks {missing}")
+            if self.high_freq_factor == self.low_freq_factor:
+                raise ConfigError("rope_scaling: high_freq_factor equals low_freq_factor")
+        if self.factor <= 0:
+            raise ConfigError("rope_scaling.factor must be positive")
+
+    def to_dict(self) -> dict[str, Any]:
+        d: dict[str, Any] = {"rope_type": self.rope_type, "factor": self.factor}
+        for k in ("low_freq_factor", "high_freq_factor", "original_max_position_embeddings"):
+            if getattr(self, k) is not None:
+                d[k] = getattr(self, k)
+        return d
+
+
+def _opt(d: dict[str, Any], key: str, cast: Callable[[Any], Any]):
+    return cast(d[key]) if d.get(key) is not None else None
+
+
+@dataclass(frozen=True)
+class LlamaConfig:
+    """The keys of a Llama ``config.json`` that the forward path consumes
+    (tokasaurus/model/llama.py:123-159 heads, :301 intermediate, :437 vocab,
+    :48 eps, :563 table length, :842-845 tie).  ``head_dim`` is derived, as at
+    llama.py:158-159; ``attention_bias``, ``mlp_bias``, ``hidden_act`` and
+    ``torch_dtype`` are not consulted there and are ignored here as well.
+    """
+
+    model_type: str
+    hidden_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    num_hidden_layers: int
+    intermediate_size: int
+    vocab_size: int
+    rms_norm_eps: float
+    max_position_embeddings: int
+    rope_theta: float
+    rope_scaling: RopeScaling | None = None
+    tie_word_embeddings: bool = False
+    eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+
+    REQUIRED = (
+        "hidden_size",
+        "num_attention_heads",
+        "num_hidden_layers",
+        "intermediate_size",
+        "vocab_size",
+        "rms_norm_eps",
+        "max_position_embeddings",
+        "rope_theta",
+    )
+
+    @property
+    def head_dim(self) -> int:
+        return self.hidden_size // self.num_attention_heads
+
+    @classmethod
+    def from_dict(cls, d: dict[str, Any]) -> "LlamaConfig":
+        missing = [k for k in cls.REQUIRED if k not in d]
+        if missing:
+            raise ConfigError(f"config.json lacks required keys: {missing}")
+        eos = d.get("eos_token_id")
+        if eos is None:
+            eos_ids: tuple[int, ...] = ()
+        elif isinstance(eos, int):
+            eos_ids = (eos,)
+        else:
+            eos_ids = tuple(int(e) for e in eos)
+        cfg = cls(
+            model_type=str(d.get("model_type", "llama")),
+            hidden_size=int(d["hidden_size"]),
+            num_attention_heads=int(d["num_attention_heads"]),
+            num_key_value_heads=int(d.get("num_key_value_heads") or d["num_attention_heads"]),
+            num_hidden_layers=int(d["num_hidden_layers"]),
+            intermediate_size=int(d["intermediate_size"]),
+            vocab_size=int(d["vocab_size"]),
+            rms_norm_eps=float(d["rms_norm_eps"]),
+            max_position_embeddings=int(d["max_position_embeddings"]),
+            rope_theta=float(d["rope_theta"]),
+            rope_scaling=RopeScaling.from_dict(d.get("rope_scaling")),
+            tie_word_embeddings=bool(d.get("tie_word_embeddings", False)),
+            eos_token_ids=eos_ids,
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        for name in (
+            "hidden_size",
+            "num_attention_heads",
+            "num_key_value_heads",
+            "num_hidden_layers",
+            "intermediate_size",
+            "vocab_size",
+            "max_position_embeddings",
+        ):
+            if getattr(self, name) <= 0:
+                raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.hidden_size % self.num_attention_heads:
+            raise ConfigError(
+                f"hidden_size {self.hidden_size} is not divisible by "
+                f"num_attention_heads {self.num_attention_heads}"
+            )
+        if self.num_attention_heads % self.num_key_value_heads:
+            raise ConfigError(
+                f"num_attention_heads {self.num_attention_heads} is not a multiple of "
+                f"num_key_value_heads {self.num_key_value_heads}"
+            )
+        if self.head_dim % 2:
+            raise ConfigError(f"head_dim {self.head_dim} must be even for the rotary pairing")
+        if not self.rms_norm_eps > 0:
+            raise ConfigError("rms_norm_eps must be positive")
+        if not self.rope_theta > 0:
+            raise ConfigError("rope_theta must be positive")
+
+    def to_dict(self) -> dict[str, Any]:
+        d: dict[str, Any] = {
+            "architectures": ["LlamaForCausalLM"],
+            "model_type": self.model_type,
+            "hidden_size": self.hidden_size,
+            "num_attention_heads": self.num_attention_heads,
+            "num_key_value_heads": self.num_key_value_heads,
+            "num_hidden_layers": self.num_hidden_layers,
+            "intermediate_size": self.intermediate_size,
+            "vocab_size": self.vocab_size,
+            "rms_norm_eps": self.rms_norm_eps,
+            "max_position_embeddings": self.max_position_embeddings,
+            "rope_theta": self.rope_theta,
+            "rope_scaling": self.rope_scaling.to_dict() if self.rope_scaling else None,
+            "tie_word_embeddings": self.tie_word_embeddings,
+        }
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d
+
+    def with_rope_scaling(self, scaling: dict[str, Any] | None) -> "LlamaConfig":
+        """The command line's ``rope_scaling='<json>'`` replaces the file's value
+        (tokasaurus/model/utils.py:353-354, tokasaurus/model/llama.py:785-786)."""
+        from dataclasses import replace
+
+        return replace(self, rope_scaling=RopeScaling.from_dict(scaling))
+
+
+def read_config_json(model_dir: str | Path) -> dict[str, Any]:
+    path = Path(model_dir) / "config.json"
+    if not path.is_file():
+        raise FileNotFoundError(f"no config.json in model folder {model_dir}")
+    d = json.loads(path.read_text())
+    gen = Path(model_dir) / "generation_config.json"
+    if gen.is_file() and "eos_token_id" not in d:
+        # tokasaurus/utils.py:447-457 takes the end-of-sequence ids from here
+        g = json.loads(gen.read_text())
+        if g.get("eos_token_id") is not None:
+            d["eos_token_id"] = g["eos_token_id"]
+    return d

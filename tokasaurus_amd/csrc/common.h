@@ -1,0 +1,92 @@
+// Shared helpers of the gfx950 kernel library: element types, reductions over a
+// 64-wide wavefront, error reporting to the Python side.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#define TK_WAVE 64
+
+enum TkDtype { TK_F32 = 0, TK_BF16 = 1 };
+
+typedef __hip_bfloat16 bf16_t;
+
+// Every entry point returns 0 or a negative code; the text is read with tk_last_error().
+void tk_set_error(const char* fmt, ...);
+
+#define TK_REQUIRE(cond, ...)        \
+  do {                               \
+    if (!(cond)) {                   \
+      tk_set_error(__VA_ARGS__);     \
+      return -1;                     \
+    }                                \
+  } while (0)
+
+#define TK_CHECK_LAUNCH(name)                                                \
+  do {                                                                       \
+    hipError_t e__ = hipGetLastError();                                      \
+    if (e__ != hipSuccess) {                                                 \
+      tk_set_error("%s: launch failed: %s", name, hipGetErrorString(e__));   \
+      return -2;                                                             \
+    }                                                                        \
+  } while (0)
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T v);
+template <>
+__device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return __bfloat162float(v); }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return __float2bfloat16(v); }
+
+// Round a 32-bit value to the storage type and back: the place where the
+// reference's tensors are materialised in the engine dtype.
+template <typename T>
+__device__ __forceinline__ float round_to(float v) { return to_f32<T>(from_f32<T>(v)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = TK_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TK_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = TK_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, TK_WAVE));
+  return v;
+}
+
+// Sum over a workgroup of up to 1024 threads; every thread gets the result.
+// `scratch` holds at least 16 floats of LDS; the order of the additions is fixed.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (TK_WAVE - 1);
+  const int wave = threadIdx.x / TK_WAVE;
+  const int nwaves = (blockDim.x + TK_WAVE - 1) / TK_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & (TK_WAVE - 1);
+  const int wave = threadIdx.x / TK_WAVE;
+  const int nwaves = (blockDim.x + TK_WAVE - 1) / TK_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int w = 1; w < nwaves; ++w) total = fmaxf(total, scratch[w]);
+  return total;
+}

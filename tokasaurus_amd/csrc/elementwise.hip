@@ -1,0 +1,265 @@
+// Memory-bound kernels of the step: embedding gather, RMSNorm, SwiGLU, row
+// gather, the rotary tables, and rotation fused with the append to the paged cache.
+// Every kernel is a template over the storage type (float or bfloat16) and
+// computes in 32-bit.
+#include "common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512];
+
+void tk_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* tk_last_error() { return g_error; }
+
+extern "C" int tk_abi_version() { return 3; }
+
+// --------------------------------------------------------------------------
+// embedding: out[t, :] = table[id_t, :]; id_t < 0 names slot -id_t-1 of `last_token`
+// (the token the sampler wrote there in the step before).
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const int* __restrict__ last_token,
+                                    const T* __restrict__ table, T* __restrict__ out, int hidden,
+                                    int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  if (id < 0) id = last_token[-id - 1];
+  id = min(max(id, 0), vocab - 1);
+  const T* src = table + (size_t)id * hidden;
+  T* dst = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int tk_embed_gather(int dt, const int* ids, const int* last_token, const void* table,
+                               void* out, int n_tokens, int hidden, int vocab, hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes %d %d %d", n_tokens,
+             hidden, vocab);
+  if (n_tokens == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, ids,
+                       last_token, (const float*)table, (float*)out, hidden, vocab);
+  else
+    hipLaunchKernelGGL(embed_gather_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, ids,
+                       last_token, (const bf16_t*)table, (bf16_t*)out, hidden, vocab);
+  TK_CHECK_LAUNCH("embed_gather");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// RMSNorm: statistics in 32-bit, the normalised value rounded to the storage
+// type, then multiplied by the weight and rounded again.  The weight is of the
+// storage type, or 32-bit when `w_f32` (then the product is rounded once more only).
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, const void* __restrict__ w, int w_f32,
+                               T* __restrict__ out, int hidden, float eps) {
+  __shared__ float red[16];
+  const T* row = x + (size_t)blockIdx.x * hidden;
+  T* orow = out + (size_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = to_f32<T>(row[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float rstd = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float n = round_to<T>(to_f32<T>(row[i]) * rstd);
+    float wi = w_f32 ? ((const float*)w)[i] : to_f32<T>(((const T*)w)[i]);
+    orow[i] = from_f32<T>(wi * n);
+  }
+}
+
+extern "C" int tk_rmsnorm(int dt, const void* x, const void* w, int w_f32, void* out, int rows,
+                          int hidden, float eps, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && hidden > 0, "rmsnorm: bad sizes %d %d", rows, hidden);
+  if (rows == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)x, w,
+                       w_f32, (float*)out, hidden, eps);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)x,
+                       w, w_f32, (bf16_t*)out, hidden, eps);
+  TK_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// SwiGLU on a fused [rows, 2*inter] product laid out [gate | up]:
+// out = round(round(silu(gate)) * up).
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+  const T* g = gu + (size_t)blockIdx.x * 2 * inter;
+  const T* u = g + inter;
+  T* o = out + (size_t)blockIdx.x * inter;
+  for (int i = threadIdx.x; i < inter; i += blockDim.x) {
+    float gv = to_f32<T>(g[i]);
+    float s = round_to<T>(gv / (1.0f + expf(-gv)));
+    o[i] = from_f32<T>(s * to_f32<T>(u[i]));
+  }
+}
+
+extern "C" int tk_swiglu(int dt, const void* gate_up, void* out, int rows, int inter,
+                         hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && inter > 0, "swiglu: bad sizes %d %d", rows, inter);
+  if (rows == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(swiglu_kernel<float>, dim3(rows), dim3(256), 0, stream,
+                       (const float*)gate_up, (float*)out, inter);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream,
+                       (const bf16_t*)gate_up, (bf16_t*)out, inter);
+  TK_CHECK_LAUNCH("swiglu");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// gather_rows: out[i, :] = src[idx[i], :]   (src rows `src_stride` elements apart)
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void gather_rows_kernel(const T* __restrict__ src, int src_stride,
+                                   const int* __restrict__ idx, T* __restrict__ out, int width) {
+  const T* s = src + (size_t)idx[blockIdx.x] * src_stride;
+  T* o = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = s[i];
+}
+
+extern "C" int tk_gather_rows(int dt, const void* src, int src_stride, const int* idx, void* out,
+                              int n, int width, hipStream_t stream) {
+  TK_REQUIRE(n >= 0 && width > 0 && src_stride >= width, "gather_rows: bad sizes %d %d %d", n,
+             width, src_stride);
+  if (n == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(n), dim3(256), 0, stream, (const float*)src,
+                       src_stride, idx, (float*)out, width);
+  else
+    hipLaunchKernelGGL(gather_rows_kernel<bf16_t>, dim3(n), dim3(256), 0, stream,
+                       (const bf16_t*)src, src_stride, idx, (bf16_t*)out, width);
+  TK_CHECK_LAUNCH("gather_rows");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// Rotary tables: cos/sin[p, j] = cos/sin(p * inv_freq[j]) for j < half, 32-bit.
+// --------------------------------------------------------------------------
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __restrict__ cos_t,
+                                  float* __restrict__ sin_t, int n_pos, int half) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_pos * half) return;
+  const int p = i / half, j = i % half;
+  const float angle = (float)p * inv_freq[j];
+  cos_t[i] = cosf(angle);
+  sin_t[i] = sinf(angle);
+}
+
+extern "C" int tk_rope_table(const float* inv_freq, float* cos_t, float* sin_t, int n_pos, int half,
+                             hipStream_t stream) {
+  TK_REQUIRE(n_pos > 0 && half > 0, "rope_table: bad sizes %d %d", n_pos, half);
+  const long total = (long)n_pos * half;
+  TK_REQUIRE(total < (1l << 31), "rope_table: table of %ld entries is too large", total);
+  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                     inv_freq, cos_t, sin_t, n_pos, half);
+  TK_CHECK_LAUNCH("rope_table");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// rope_append: for each token rotate its query heads in place, rotate its key
+// heads and store them, and store its value heads, in the token's page.
+//   qkv row: [nq*d | nkv*d | nkv*d]  (only the first part when !write_cache)
+//   K pages: [page][kv head][P][d]       V pages: [page][kv head][d][P]
+// Lane j pairs with lane j + d/2; the rotation is computed in 32-bit.
+// When cos_t is null the heads are stored unrotated (no position encoding).
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
+                                   const int* __restrict__ positions,
+                                   const int* __restrict__ token_req,
+                                   const int* __restrict__ block_table, int table_stride,
+                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                   T* __restrict__ kcache, T* __restrict__ vcache, int nq, int nkv,
+                                   int d, int P, int write_cache) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = d / 2;
+  T* row = qkv + (size_t)t * row_stride;
+  const float* c = cos_t ? cos_t + (size_t)pos * half : nullptr;
+  const float* s = sin_t ? sin_t + (size_t)pos * half : nullptr;
+
+  // queries, in place
+  for (int i = threadIdx.x; i < nq * half; i += blockDim.x) {
+    const int h = i / half, j = i % half;
+    T* x = row + h * d;
+    const float x1 = to_f32<T>(x[j]), x2 = to_f32<T>(x[j + half]);
+    const float cj = c ? c[j] : 1.f, sj = s ? s[j] : 0.f;
+    x[j] = from_f32<T>(x1 * cj - x2 * sj);
+    x[j + half] = from_f32<T>(x2 * cj + x1 * sj);
+  }
+  if (!write_cache) return;
+
+  const int page = block_table[(size_t)token_req[t] * table_stride + pos / P];
+  const int p = pos % P;
+  const T* krow = row + nq * d;
+  const T* vrow = krow + nkv * d;
+  for (int i = threadIdx.x; i < nkv * half; i += blockDim.x) {
+    const int h = i / half, j = i % half;
+    const float x1 = to_f32<T>(krow[h * d + j]), x2 = to_f32<T>(krow[h * d + j + half]);
+    const float cj = c ? c[j] : 1.f, sj = s ? s[j] : 0.f;
+    T* dst = kcache + (((size_t)page * nkv + h) * P + p) * d;
+    dst[j] = from_f32<T>(x1 * cj - x2 * sj);
+    dst[j + half] = from_f32<T>(x2 * cj + x1 * sj);
+  }
+  for (int i = threadIdx.x; i < nkv * d; i += blockDim.x) {
+    const int h = i / d, e = i % d;
+    vcache[(((size_t)page * nkv + h) * d + e) * P + p] = vrow[i];
+  }
+}
+
+extern "C" int tk_rope_append(int dt, void* qkv, int row_stride, const int* positions,
+                              const int* token_req, const int* block_table, int table_stride,
+                              const float* cos_t, const float* sin_t, void* kcache, void* vcache,
+                              int n_tokens, int nq, int nkv, int d, int P, int write_cache,
+                              hipStream_t stream) {
+  TK_REQUIRE(n_tokens >= 0 && nq > 0 && nkv >= 0 && d > 0 && d % 2 == 0 && P > 0,
+             "rope_append: bad sizes tokens=%d nq=%d nkv=%d d=%d P=%d", n_tokens, nq, nkv, d, P);
+  TK_REQUIRE(row_stride >= (write_cache ? (nq + 2 * nkv) * d : nq * d),
+             "rope_append: row stride %d is shorter than the heads it holds", row_stride);
+  TK_REQUIRE(!write_cache || (kcache && vcache && block_table),
+             "rope_append: cache pointers missing");
+  if (n_tokens == 0) return 0;
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(rope_append_kernel<float>, dim3(n_tokens), dim3(256), 0, stream,
+                       (float*)qkv, row_stride, positions, token_req, block_table, table_stride,
+                       cos_t, sin_t, (float*)kcache, (float*)vcache, nq, nkv, d, P, write_cache);
+  else
+    hipLaunchKernelGGL(rope_append_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream,
+                       (bf16_t*)qkv, row_stride, positions, token_req, block_table, table_stride,
+                       cos_t, sin_t, (bf16_t*)kcache, (bf16_t*)vcache, nq, nkv, d, P, write_cache);
+  TK_CHECK_LAUNCH("rope_append");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// fill: used instead of a memset so that it may be recorded into a HIP graph.
+// --------------------------------------------------------------------------
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+extern "C" int tk_fill_u32(void* p, uint32_t value, size_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  TK_REQUIRE(n < ((size_t)1 << 40), "fill: too many elements");
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                     (uint32_t*)p, value, n);
+  TK_CHECK_LAUNCH("fill_u32");
+  return 0;
+}

@@ -1,0 +1,154 @@
+"""From a list of (request, next tokens, wanted places) to the arrays a step runs on.
+
+The layout follows the reference's ``seqs_to_input``
+(tokasaurus/manager/input_building.py:151-320): tokens request by request,
+prompt portions first and single decoded tokens after them, a position per
+token, the rows whose logits are wanted, and per request its pages.  Example
+with page size 4: request A holds 4 tokens and brings 6 more with table
+[5, 2, 9]; request B decodes at position 7 with table [7, 1].  Then positions
+are [4..9, 7], token_req is [0]*6 + [1], q_start [0, 6, 7], kv_len [10, 8] and
+the block table [[5, 2, 9], [7, 1, -1]].
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from tokasaurus_amd.parts.base import StepContext
+
+FROM_SLOT = None  # tokens=None: the one token is the slot's last sampled token
+
+
+@dataclass
+class StepEntry:
+    request_id: str
+    tokens: list[int] | None
+    want: list[int] = field(default_factory=list)
+
+
+@dataclass
+class PlannedEntry:
+    """An entry resolved against the cache manager."""
+
+    request_id: str
+    tokens: list[int] | None
+    want: list[int]
+    slot: int
+    start: int  # tokens the request holds before this step
+    tables: list[list[int]]  # per cache group
+
+    @property
+    def q_len(self) -> int:
+        return 1 if self.tokens is None else len(self.tokens)
+
+
+@dataclass
+class HostBatch:
+    """The step's arrays on the host, entries reordered (portions first)."""
+
+    order: list[int]  # order[i] = index in the caller's list of the i-th request of the batch
+    token_ids: list[int]
+    positions: list[int]
+    token_req: list[int]
+    q_start: list[int]
+    kv_len: list[int]
+    slots: list[int]
+    want_rows: list[int]  # in the caller's order of entries and of `want`
+    block_tables: list[list[list[int]]]  # per group, per request (batch order), padded with -1
+    num_portions: int  # requests with more than one token come first
+
+
+def layout(entries: list[PlannedEntry], vocab_size: int, num_groups: int) -> HostBatch:
+    for e in entries:
+        if e.tokens is not None:
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.request_id!r} brings no tokens")
+            bad = [t for t in e.tokens if not 0 <= t < vocab_size]
+            if bad:
+                raise ValueError(f"request {e.request_id!r}: token ids {bad[:4]} outside the vocabulary of {vocab_size}")
+        for w in e.want:
+            if not 0 <= w < e.q_len:
+                raise ValueError(f"request {e.request_id!r}: wanted place {w} outside its {e.q_len} tokens")
+    if len({e.request_id for e in entries}) != len(entries):
+        raise ValueError("a request appears twice in one step")
+    order = [i for i, e in enumerate(entries) if e.q_len > 1] + [i for i, e in enumerate(entries) if e.q_len == 1]
+    num_portions = sum(1 for e in entries if e.q_len > 1)
+    token_ids: list[int] = []
+    positions: list[int] = []
+    token_req: list[int] = []
+    q_start = [0]
+    kv_len: list[int] = []
+    slots: list[int] = []
+    first_row = {}
+    for r, i in enumerate(order):
+        e = entries[i]
+        first_row[i] = len(token_ids)
+        if e.tokens is None:
+            token_ids.append(-(e.slot + 1))
+        else:
+            token_ids.extend(e.tokens)
+        positions.extend(range(e.start, e.start + e.q_len))
+        token_req.extend([r] * e.q_len)
+        q_start.append(len(token_ids))
+        kv_len.append(e.start + e.q_len)
+        slots.append(e.slot)
+    want_rows = [first_row[i] + w for i, e in enumerate(entries) for w in e.want]
+    block_tables = []
+    for g in range(num_groups):
+        width = max((len(entries[i].tables[g]) for i in order), default=0)
+        width = max(width, 1)
+        block_tables.append([entries[i].tables[g] + [-1] * (width - len(entries[i].tables[g])) for i in order])
+    return HostBatch(order, token_ids, positions, token_req, q_start, kv_len, slots, want_rows, block_tables, num_portions)
+
+
+def to_device(hb: HostBatch, dtype: torch.dtype, device: torch.device, last_token: torch.Tensor | None):
+    """One packed int32 upload; returns the context, the wanted rows and the block tables."""
+    n, r = len(hb.token_ids), len(hb.kv_len)
+    flat: list[int] = []
+    spans = {}
+
+    def put(name: str, values: list[int]) -> None:
+        spans[name] = (len(flat), len(values))
+        flat.extend(values)
+
+    put("token_ids", hb.token_ids)
+    put("positions", hb.positions)
+    put("token_req", hb.token_req)
+    put("q_start", hb.q_start)
+    put("kv_len", hb.kv_len)
+    put("slots", hb.slots)
+    put("want_rows", hb.want_rows)
+    widths = []
+    for g, table in enumerate(hb.block_tables):
+        widths.append(len(table[0]) if table else 1)
+        put(f"table{g}", [p for row in table for p in row])
+    packed = torch.tensor(flat, dtype=torch.int32).to(device, non_blocking=False)
+
+    def view(name: str) -> torch.Tensor:
+        a, m = spans[name]
+        return packed[a : a + m]
+
+    q_lens = [hb.q_start[i + 1] - hb.q_start[i] for i in range(r)]
+    ctx = StepContext(
+        num_tokens=n,
+        num_requests=r,
+        dtype=dtype,
+        device=device,
+        token_ids=view("token_ids"),
+        positions=view("positions"),
+        token_req=view("token_req"),
+        q_start=view("q_start"),
+        kv_len=view("kv_len"),
+        slots=view("slots"),
+        host_q_start=hb.q_start,
+        host_kv_len=hb.kv_len,
+        host_slots=hb.slots,
+        last_token=last_token,
+        max_q_len=max(q_lens, default=0),
+        max_kv_len=max(hb.kv_len, default=0),
+    )
+    ctx.extras["num_portions"] = hb.num_portions
+    tables = [view(f"table{g}").view(r, widths[g]) if r else view(f"table{g}").view(0, 1) for g in range(len(hb.block_tables))]
+    return ctx, view("want_rows"), tables

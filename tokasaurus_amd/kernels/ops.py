@@ -1,0 +1,336 @@
+"""Typed Python wrappers of the kernel library: they check shapes, types and
+devices on the host (a kernel is never launched on operands it was not written
+for), allocate outputs with torch, and launch on torch's current stream, so a
+step can be recorded into a HIP graph.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from tokasaurus_amd.kernels.library import KernelError, call
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 storage, not {dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU; there is no CPU path")
+
+
+def _i32(t: torch.Tensor, name: str) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
+
+
+def embed_gather(
+    ids: torch.Tensor, table: torch.Tensor, last_token: torch.Tensor | None = None
+) -> torch.Tensor:
+    """out[t] = table[ids[t]]; ids[t] < 0 reads the token from last_token[-ids[t]-1]."""
+    _gpu(ids, table, last_token)
+    _i32(ids, "ids")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [V, H]")
+    if last_token is not None:
+        _i32(last_token, "last_token")
+    n = ids.numel()
+    vocab, hidden = table.shape
+    out = torch.empty((n, hidden), dtype=table.dtype, device=table.device)
+    call(
+        "tk_embed_gather",
+        dtype_code(table.dtype),
+        ids.data_ptr(),
+        last_token.data_ptr() if last_token is not None else None,
+        table.data_ptr(),
+        out.data_ptr(),
+        n,
+        hidden,
+        vocab,
+        _stream(),
+    )
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    _gpu(x, weight)
+    _need(x.dim() == 2 and x.is_contiguous(), "rmsnorm input must be contiguous [rows, H]")
+    rows, hidden = x.shape
+    _need(weight.shape == (hidden,) and weight.is_contiguous(), "rmsnorm weight must be [H]")
+    _need(
+        weight.dtype in (x.dtype, torch.float32),
+        f"rmsnorm weight is {weight.dtype}, expected {x.dtype} or float32",
+    )
+    out = torch.empty_like(x)
+    w_f32 = 1 if (weight.dtype == torch.float32 and x.dtype != torch.float32) else 0
+    call(
+        "tk_rmsnorm",
+        dtype_code(x.dtype),
+        x.data_ptr(),
+        weight.data_ptr(),
+        w_f32,
+        out.data_ptr(),
+        rows,
+        hidden,
+        float(eps),
+        _stream(),
+    )
+    return out
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """[rows, 2I] laid out [gate | up] -> silu(gate) * up, [rows, I]."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0,
+          "swiglu input must be contiguous [rows, 2I]")
+    rows, two_i = gate_up.shape
+    out = torch.empty((rows, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    call("tk_swiglu", dtype_code(gate_up.dtype), gate_up.data_ptr(), out.data_ptr(), rows,
+         two_i // 2, _stream())
+    return out
+
+
+def gather_rows(src: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+    """out[i] = src[idx[i]] for a 2-d ``src`` whose rows may be strided."""
+    _gpu(src, idx)
+    _i32(idx, "row indices")
+    _need(src.dim() == 2 and src.stride(1) == 1, "gather_rows source must be 2-d with unit inner stride")
+    n, width = idx.numel(), src.shape[1]
+    out = torch.empty((n, width), dtype=src.dtype, device=src.device)
+    call("tk_gather_rows", dtype_code(src.dtype), src.data_ptr(), src.stride(0), idx.data_ptr(),
+         out.data_ptr(), n, width, _stream())
+    return out
+
+
+def rope_table(inv_freq: torch.Tensor, n_pos: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos and sin of position * inv_freq, each [n_pos, d/2] in 32-bit."""
+    _gpu(inv_freq)
+    _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and inv_freq.is_contiguous(),
+          "inv_freq must be contiguous float32 [d/2]")
+    half = inv_freq.numel()
+    cos = torch.empty((n_pos, half), dtype=torch.float32, device=inv_freq.device)
+    sin = torch.empty_like(cos)
+    call("tk_rope_table", inv_freq.data_ptr(), cos.data_ptr(), sin.data_ptr(), n_pos, half, _stream())
+    return cos, sin
+
+
+def rope_append(
+    qkv: torch.Tensor,
+    positions: torch.Tensor,
+    token_req: torch.Tensor,
+    block_table: torch.Tensor | None,
+    cos: torch.Tensor | None,
+    sin: torch.Tensor | None,
+    kcache: torch.Tensor | None,
+    vcache: torch.Tensor | None,
+    nq: int,
+    nkv: int,
+    head_dim: int,
+    page_size: int,
+    write_cache: bool = True,
+) -> None:
+    """Rotate the query heads of ``qkv`` in place; rotate the key heads and store
+    them and the value heads in each token's page.
+
+    ``kcache`` is [pages, nkv, P, d], ``vcache`` is [pages, nkv, d, P] (values
+    transposed inside a page).  ``block_table`` is [requests, width] int32.
+    """
+    _gpu(qkv, positions, token_req, block_table, cos, sin, kcache, vcache)
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be 2-d with unit inner stride")
+    n = qkv.shape[0]
+    _i32(positions, "positions")
+    _i32(token_req, "token_req")
+    _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
+    half = head_dim // 2
+    if cos is not None:
+        _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+              and cos.shape == sin.shape and cos.shape[1] == half and cos.is_contiguous()
+              and sin.is_contiguous(), "cos/sin tables must be contiguous float32 [positions, d/2]")
+    table_stride = 0
+    if write_cache:
+        _need(block_table is not None and kcache is not None and vcache is not None,
+              "rope_append needs the cache and the block table to write")
+        _i32(block_table, "block_table")
+        _need(block_table.dim() == 2, "block_table must be [requests, width]")
+        table_stride = block_table.stride(0)
+        pages = kcache.shape[0]
+        _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
+              f"key pages must be contiguous [pages, {nkv}, {page_size}, {head_dim}], got {tuple(kcache.shape)}")
+        _need(tuple(vcache.shape) == (pages, nkv, head_dim, page_size) and vcache.is_contiguous(),
+              f"value pages must be contiguous [pages, {nkv}, {head_dim}, {page_size}], got {tuple(vcache.shape)}")
+        _need(kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype, "cache dtype differs from qkv")
+    call(
+        "tk_rope_append",
+        dtype_code(qkv.dtype),
+        qkv.data_ptr(),
+        qkv.stride(0),
+        positions.data_ptr(),
+        token_req.data_ptr(),
+        block_table.data_ptr() if write_cache else None,
+        table_stride,
+        cos.data_ptr() if cos is not None else None,
+        sin.data_ptr() if sin is not None else None,
+        kcache.data_ptr() if write_cache else None,
+        vcache.data_ptr() if write_cache else None,
+        n,
+        nq,
+        nkv if write_cache else 0,
+        head_dim,
+        page_size,
+        1 if write_cache else 0,
+        _stream(),
+    )
+
+
+def gemm_generic(
+    a: torch.Tensor,
+    w: torch.Tensor,
+    residual: torch.Tensor | None = None,
+    out_f32: bool = False,
+) -> torch.Tensor:
+    """a [M, K] times w [N, K] transposed (+ residual [M, N]), 32-bit multiply-adds."""
+    _gpu(a, w, residual)
+    _need(a.dim() == 2 and a.stride(1) == 1, "gemm: A must be 2-d with unit inner stride")
+    _need(w.dim() == 2 and w.is_contiguous(), "gemm: W must be contiguous [N, K]")
+    _need(a.dtype == w.dtype, f"gemm: A is {a.dtype} but W is {w.dtype}")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k, f"gemm: A has K={k} but W has K={w.shape[1]}")
+    out_dtype = torch.float32 if out_f32 else a.dtype
+    out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    ldr = 0
+    if residual is not None:
+        _need(not out_f32, "gemm: a residual cannot be combined with 32-bit output")
+        _need(residual.shape == (m, n) and residual.stride(1) == 1 and residual.dtype == a.dtype,
+              "gemm: residual must be [M, N] of the operand type")
+        ldr = residual.stride(0)
+    call(
+        "tk_gemm_generic",
+        dtype_code(a.dtype),
+        a.data_ptr(),
+        a.stride(0),
+        w.data_ptr(),
+        out.data_ptr(),
+        n,
+        residual.data_ptr() if residual is not None else None,
+        ldr,
+        m,
+        n,
+        k,
+        1 if out_f32 else 0,
+        _stream(),
+    )
+    return out
+
+
+def paged_attention_generic(
+    q: torch.Tensor,
+    kcache: torch.Tensor,
+    vcache: torch.Tensor,
+    block_table: torch.Tensor,
+    token_req: torch.Tensor,
+    positions: torch.Tensor,
+    nq: int,
+    nkv: int,
+    head_dim: int,
+    page_size: int,
+    window: int = 0,
+    scale: float | None = None,
+) -> torch.Tensor:
+    """Attention of every token over its request's pages (see rope_append for
+    the page layout).  ``q`` is 2-d, its first nq*d columns are the query heads."""
+    _gpu(q, kcache, vcache, block_table, token_req, positions)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * head_dim,
+          "attention: q must be 2-d with unit inner stride and nq*d leading columns")
+    n = q.shape[0]
+    _i32(block_table, "block_table")
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    _need(block_table.dim() == 2, "block_table must be [requests, width]")
+    _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
+    pages = kcache.shape[0]
+    _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
+          "attention: key pages must be contiguous [pages, nkv, P, d]")
+    _need(tuple(vcache.shape) == (pages, nkv, head_dim, page_size) and vcache.is_contiguous(),
+          "attention: value pages must be contiguous [pages, nkv, d, P]")
+    _need(kcache.dtype == q.dtype and vcache.dtype == q.dtype, "attention: cache dtype differs from q")
+    out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
+    call(
+        "tk_paged_attention_generic",
+        dtype_code(q.dtype),
+        q.data_ptr(),
+        q.stride(0),
+        out.data_ptr(),
+        out.stride(0),
+        kcache.data_ptr(),
+        vcache.data_ptr(),
+        block_table.data_ptr(),
+        block_table.stride(0),
+        token_req.data_ptr(),
+        positions.data_ptr(),
+        n,
+        nq,
+        nkv,
+        head_dim,
+        page_size,
+        int(window),
+        float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
+        _stream(),
+    )
+    return out
+
+
+def sample(
+    logits: torch.Tensor,
+    temperature: torch.Tensor,
+    uniform: torch.Tensor,
+    slots: torch.Tensor | None = None,
+    last_token: torch.Tensor | None = None,
+    want_logprobs: bool = True,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Token ids (int32) and their log-probabilities for each row of ``logits``."""
+    _gpu(logits, temperature, uniform, slots, last_token)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
+          "sample: logits must be float32 [rows, vocab]")
+    rows, vocab = logits.shape
+    for t, name in ((temperature, "temperature"), (uniform, "uniform")):
+        _need(t.dtype == torch.float32 and t.numel() == rows and t.is_contiguous(),
+              f"sample: {name} must be float32 [rows]")
+    if slots is not None or last_token is not None:
+        _need(slots is not None and last_token is not None, "sample: slots and last_token go together")
+        _i32(slots, "slots")
+        _i32(last_token, "last_token")
+        _need(slots.numel() == rows, "sample: one slot a row")
+    ids = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    logprobs = torch.empty((rows,), dtype=torch.float32, device=logits.device) if want_logprobs else None
+    call(
+        "tk_sample",
+        logits.data_ptr(),
+        logits.stride(0) if rows > 0 else vocab,
+        rows,
+        vocab,
+        temperature.data_ptr(),
+        uniform.data_ptr(),
+        slots.data_ptr() if slots is not None else None,
+        last_token.data_ptr() if last_token is not None else None,
+        ids.data_ptr(),
+        logprobs.data_ptr() if logprobs is not None else None,
+        _stream(),
+    )
+    return ids, logprobs

@@ -1,0 +1,72 @@
+"""A causal language model built from a ``ModelSpec``: embedding, the blocks in
+run order, final norm and head (the skeleton of tokasaurus/model/llama.py:521-582,
+603-667 with the architecture taken out of it)."""
+
+from __future__ import annotations
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.models.spec import ModelSpec
+from tokasaurus_amd.parts.base import BLOCKS, CacheNeed, CacheView, Part, StateNeed, StepContext, TensorSpec
+from tokasaurus_amd.parts.block import build_with_shared
+from tokasaurus_amd.parts.embedding import LMHead, TokenEmbedding
+from tokasaurus_amd.parts.linear import Placer
+
+
+class CausalLM:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        self.shared: dict = {}
+        self.embedding = TokenEmbedding(spec.vocab_size, spec.hidden_size, spec.embedding_name)
+        self.blocks = [build_with_shared(BLOCKS, b, self.shared) for b in spec.layers]
+        self.head = LMHead(spec.vocab_size, spec.hidden_size, spec.head_name, spec.final_norm)
+        self.dtype: torch.dtype | None = None
+        self.device: torch.device | None = None
+        self.weight_bytes = 0
+
+    # ---- tensors
+    def parts(self) -> list[Part]:
+        return [self.embedding, *self.blocks, self.head]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        seen: dict[str, TensorSpec] = {}
+        for part in self.parts():
+            for s in part.tensor_specs():
+                if s.name in seen and seen[s.name].shape != s.shape:
+                    raise ValueError(f"tensor {s.name} is wanted with shapes {seen[s.name].shape} and {s.shape}")
+                seen.setdefault(s.name, s)
+        return list(seen.values())
+
+    def load(self, tensors: dict[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
+        placer = Placer(dtype, device)
+        for part in self.parts():
+            part.load(tensors, placer)
+        self.dtype, self.device = dtype, device
+        self.weight_bytes = placer.bytes_placed()
+
+    # ---- what the cache manager must provide, one item per run entry
+    def cache_needs(self) -> list[CacheNeed | None]:
+        return [self.blocks[e.layer].mixer.cache_need() for e in self.spec.run_order]
+
+    def state_needs(self) -> list[StateNeed | None]:
+        return [self.blocks[e.layer].mixer.state_need() for e in self.spec.run_order]
+
+    # ---- one step
+    def forward(
+        self,
+        ctx: StepContext,
+        caches: list[CacheView | None],
+        states: list[torch.Tensor | None],
+        want_rows: torch.Tensor,
+    ) -> torch.Tensor:
+        """Run the batch of ``ctx`` and return logits [len(want_rows), vocab] in 32-bit."""
+        x = self.embedding.forward(ctx)
+        last = len(self.spec.run_order) - 1
+        for i, entry in enumerate(self.spec.run_order):
+            rows = want_rows if i == last else None
+            x = self.blocks[entry.layer].forward(x, ctx, caches[i], states[i], rows)
+        if last < 0:
+            x = ops.gather_rows(x, want_rows)
+        return self.head.forward(x)

@@ -1,0 +1,100 @@
+"""Grouped-query attention over the paged cache
+(tokasaurus/model/llama.py:96-287, tokasaurus/model/attention_utils.py:87-175).
+
+q, k and v are one stacked product; the rotation of q and k is fused with the
+append of k and v to the request's pages; one attention call then serves
+prompt portions and single decoded tokens alike, each token reading the keys
+at positions up to its own (bottom-right aligned causal mask), optionally only
+the last ``window`` of them.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import (
+    MIXERS,
+    POSITION_ENCODINGS,
+    CacheNeed,
+    CacheView,
+    Mixer,
+    PartSpec,
+    StepContext,
+    TensorSpec,
+)
+from tokasaurus_amd.parts.linear import Linear, Placer
+
+
+@MIXERS.register("paged_attention")
+class PagedAttention(Mixer):
+    def __init__(
+        self,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        names: dict[str, str],
+        position: PartSpec | None = None,
+        window: int = 0,
+        shared: dict | None = None,
+    ):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.window = int(window)
+        self.scale = 1.0 / math.sqrt(head_dim)
+        self.qkv = Linear(
+            hidden_size,
+            [names["q"], names["k"], names["v"]],
+            [num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
+        )
+        self.out = Linear(num_heads * head_dim, [names["o"]], [hidden_size])
+        self.position = None
+        if position is not None:
+            shared = shared if shared is not None else {}
+            self.position = shared.setdefault(("position", position), POSITION_ENCODINGS.build(position))
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return self.qkv.tensor_specs() + self.out.tensor_specs()
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.qkv.load(tensors, placer)
+        self.out.load(tensors, placer)
+        if self.position is not None:
+            self.position.prepare(placer.device)
+
+    def forward(
+        self,
+        h: torch.Tensor,
+        residual: torch.Tensor,
+        ctx: StepContext,
+        cache: CacheView | None,
+        state: torch.Tensor | None,
+        rows: torch.Tensor | None,
+    ) -> torch.Tensor:
+        assert cache is not None, "paged attention needs a cache"
+        nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        # an entry that reads another entry's cache computes only its queries
+        qkv = self.qkv(h, rows=None if cache.writable else nq * d)
+        cos = self.position.cos if self.position is not None else None
+        sin = self.position.sin if self.position is not None else None
+        ops.rope_append(
+            qkv, ctx.positions, ctx.token_req, cache.block_table, cos, sin,
+            cache.keys, cache.values, nq, nkv, d, cache.page_size, write_cache=cache.writable,
+        )
+        attn = ops.paged_attention_generic(
+            qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
+            nq, nkv, d, cache.page_size, window=self.window, scale=self.scale,
+        )
+        if rows is not None:
+            attn = ops.gather_rows(attn, rows)
+        return self.out(attn, residual=residual)

@@ -1,0 +1,236 @@
+"""What a part is, what a step hands to it, and the registries parts are chosen from.
+
+A model is put together from parts: a mixer (attention here), a feed-forward, norms,
+a position encoding, and the arrangement of these in a block.  A part is built from
+plain parameters (sizes, constants, the checkpoint names of its tensors); it does
+not see a model configuration and does not know which model it is in.  The
+reference hard-wires one class per role and swaps classes by subclassing
+(tokasaurus/model/llama.py:342-359, tokasaurus/model/qwen.py:11-25); here the
+roles are interfaces and the choice is data (``PartSpec``), layer by layer.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable
+
+import torch
+
+
+# --------------------------------------------------------------------------
+# descriptions of tensors, caches and state that a part needs
+# --------------------------------------------------------------------------
+
+MATRIX = "matrix"  # a projection or table of floats: engine dtype, N(0, 0.02) when random
+NORM_WEIGHT = "norm_weight"  # a norm's scale vector: 1 + N(0, 0.01) when random
+INT_TABLE = "int_table"  # integer table: kept as int32
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """One tensor a part reads from the checkpoint, by its name there."""
+
+    name: str
+    shape: tuple[int, ...]
+    kind: str = MATRIX
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Keys and values a mixer keeps per token.  Layers whose needs are equal
+    share a cache group (one page pool, one block table per request)."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0  # 0: every key is kept; > 0: only the last `window` positions are read
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size (for mixers that carry a recurrent state)."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """The choice of a part: its registered kind and its constructor parameters."""
+
+    kind: str
+    params: dict[str, Any] = field(default_factory=dict)
+
+    def __hash__(self) -> int:  # params may hold dicts; specs are compared by value
+        return hash((self.kind, repr(sorted(self.params.items(), key=lambda kv: kv[0]))))
+
+
+# --------------------------------------------------------------------------
+# what a step hands to the parts
+# --------------------------------------------------------------------------
+
+
+@dataclass
+class CacheView:
+    """The pages of one cache-owning run entry, and its group's block table for this step."""
+
+    keys: torch.Tensor  # [pages, nkv, P, d]
+    values: torch.Tensor  # [pages, nkv, d, P]
+    block_table: torch.Tensor  # [requests, width] int32, -1 where no page is held
+    page_size: int
+    writable: bool = True  # False when the entry reads another entry's cache
+
+
+@dataclass
+class StepContext:
+    """One batch: tokens of several requests, laid out request by request.
+
+    Request r owns tokens q_start[r] .. q_start[r+1]-1 at positions
+    kv_len[r] - q_len[r] .. kv_len[r] - 1.  Host copies (lists) are kept beside
+    the device arrays for parts that plan on the host.
+    """
+
+    num_tokens: int
+    num_requests: int
+    dtype: torch.dtype
+    device: torch.device
+    token_ids: torch.Tensor  # [N] int32; < 0: token is read from last_token[-id-1]
+    positions: torch.Tensor  # [N] int32
+    token_req: torch.Tensor  # [N] int32, index of each token's request in this batch
+    q_start: torch.Tensor  # [R+1] int32
+    kv_len: torch.Tensor  # [R] int32, keys of the request after this step's append
+    slots: torch.Tensor  # [R] int32, the request's state slot
+    host_q_start: list[int]
+    host_kv_len: list[int]
+    host_slots: list[int]
+    last_token: torch.Tensor | None = None  # [slots] int32, written by the sampler
+    max_q_len: int = 0
+    max_kv_len: int = 0
+    extras: dict[str, Any] = field(default_factory=dict)  # planning data of kernels, by name
+
+
+# --------------------------------------------------------------------------
+# interfaces
+# --------------------------------------------------------------------------
+
+
+class Part:
+    """Common to every part: which tensors it reads, and receiving them."""
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return []
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Any) -> None:
+        """Take this part's tensors (host tensors by checkpoint name, already
+        checked against ``tensor_specs``) and put them on the device through
+        ``placer`` (``parts.linear.Placer``: engine dtype, device, one buffer per
+        tensor) in the layout the part's kernels want."""
+
+    def children(self) -> list["Part"]:
+        return []
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Prepared once (tables on the device), then handed to the mixers that use it."""
+
+    def prepare(self, device: torch.device) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information across the tokens of a request.
+
+    ``forward`` gets the normed hidden states ``h`` [N, H], the residual stream
+    ``residual`` ([N, H], or [len(rows), H] when ``rows`` is given) and returns
+    the new residual stream ``residual + mix(h)``.  When ``rows`` (int32 indices)
+    is given only those tokens' outputs are needed (the last block of a step
+    keeps only the rows whose logits are wanted), but every token must still
+    update the cache or state.
+    """
+
+    def cache_need(self) -> CacheNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(
+        self,
+        h: torch.Tensor,
+        residual: torch.Tensor,
+        ctx: StepContext,
+        cache: CacheView | None,
+        state: torch.Tensor | None,
+        rows: torch.Tensor | None,
+    ) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Token-wise transformation: returns ``residual + ff(h)``."""
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """The arrangement of norms, a mixer and a feed-forward around the residual stream."""
+
+    mixer: Mixer
+
+    def forward(
+        self,
+        x: torch.Tensor,
+        ctx: StepContext,
+        cache: CacheView | None,
+        state: torch.Tensor | None,
+        rows: torch.Tensor | None,
+    ) -> torch.Tensor:
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------
+# registries
+# --------------------------------------------------------------------------
+
+
+class Registry:
+    """Name -> constructor for one role.  Registering a name twice is an error
+    unless ``replace=True`` (tests register toy parts)."""
+
+    def __init__(self, role: str):
+        self.role = role
+        self._entries: dict[str, Callable[..., Any]] = {}
+
+    def register(self, name: str, replace: bool = False):
+        def deco(cls):
+            if name in self._entries and not replace:
+                raise KeyError(f"{self.role} {name!r} is already registered")
+            self._entries[name] = cls
+            return cls
+
+        return deco
+
+    def build(self, spec: PartSpec, **extra: Any):
+        if spec.kind not in self._entries:
+            raise KeyError(
+                f"unknown {self.role} {spec.kind!r}; registered: {sorted(self._entries)}"
+            )
+        return self._entries[spec.kind](**spec.params, **extra)
+
+    def names(self) -> list[str]:
+        return sorted(self._entries)
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._entries
+
+
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block arrangement")

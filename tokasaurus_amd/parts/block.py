@@ -1,0 +1,77 @@
+"""Arrangements of norms, mixer and feed-forward around the residual stream.
+
+``pre_norm`` is the reference's block (tokasaurus/model/llama.py:342-359 with
+:227-230,284 and :323-325,336): each half norms its input, transforms it and adds
+the result to the stream.  In the last block of a step only the rows whose
+logits are wanted go on after the mixer (llama.py:268-278).
+"""
+
+from __future__ import annotations
+
+import inspect
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import (
+    BLOCKS,
+    FEED_FORWARDS,
+    MIXERS,
+    NORMS,
+    Block,
+    CacheView,
+    Part,
+    PartSpec,
+    StepContext,
+    TensorSpec,
+)
+from tokasaurus_amd.parts.linear import Placer
+
+
+def build_with_shared(registry, spec: PartSpec, shared: dict):
+    """Build a part; hand it the model-wide ``shared`` dict if its constructor takes one."""
+    ctor = registry._entries.get(spec.kind)
+    if ctor is not None and "shared" in inspect.signature(ctor).parameters:
+        return registry.build(spec, shared=shared)
+    return registry.build(spec)
+
+
+@BLOCKS.register("pre_norm")
+class PreNormBlock(Block):
+    def __init__(
+        self,
+        mixer_norm: PartSpec,
+        mixer: PartSpec,
+        ff_norm: PartSpec,
+        feed_forward: PartSpec,
+        shared: dict | None = None,
+    ):
+        shared = shared if shared is not None else {}
+        self.mixer_norm = build_with_shared(NORMS, mixer_norm, shared)
+        self.mixer = build_with_shared(MIXERS, mixer, shared)
+        self.ff_norm = build_with_shared(NORMS, ff_norm, shared)
+        self.feed_forward = build_with_shared(FEED_FORWARDS, feed_forward, shared)
+
+    def children(self) -> list[Part]:
+        return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [s for c in self.children() for s in c.tensor_specs()]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        for c in self.children():
+            c.load(tensors, placer)
+
+    def forward(
+        self,
+        x: torch.Tensor,
+        ctx: StepContext,
+        cache: CacheView | None,
+        state: torch.Tensor | None,
+        rows: torch.Tensor | None,
+    ) -> torch.Tensor:
+        h = self.mixer_norm.forward(x)
+        residual = x if rows is None else ops.gather_rows(x, rows)
+        x = self.mixer.forward(h, residual, ctx, cache, state, rows)
+        h = self.ff_norm.forward(x)
+        return self.feed_forward.forward(h, x)

@@ -1,0 +1,56 @@
+"""Token embedding and the language-model head.
+
+Embedding is a plain row gather without scaling (tokasaurus/model/llama.py:507-518).
+The head norms the kept rows and multiplies by the head matrix, which is the
+embedding matrix itself when the checkpoint ties them (llama.py:426-467,842-845);
+logits leave in 32-bit.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import MATRIX, NORMS, Part, PartSpec, StepContext, TensorSpec
+from tokasaurus_amd.parts.linear import Linear, Placer
+
+
+class TokenEmbedding(Part):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str):
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.name = name
+        self.table: torch.Tensor | None = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [TensorSpec(self.name, (self.vocab_size, self.hidden_size), MATRIX)]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        host = tensors[self.name]
+        self.table = placer.place(
+            ("row_major", self.name), lambda: host.to(dtype=placer.dtype).contiguous().to(placer.device)
+        )
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        return ops.embed_gather(ctx.token_ids, self.table, ctx.last_token)
+
+
+class LMHead(Part):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, norm: PartSpec):
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.norm = NORMS.build(norm)
+        self.proj = Linear(hidden_size, [name], [vocab_size])
+
+    def children(self) -> list[Part]:
+        return [self.norm]
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return self.norm.tensor_specs() + self.proj.tensor_specs()
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.norm.load(tensors, placer)
+        self.proj.load(tensors, placer)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.proj(self.norm.forward(x), out_f32=True)

@@ -1,0 +1,30 @@
+"""Dense gated feed-forward (tokasaurus/model/llama.py:290-339):
+``x + down(silu(gate(h)) * up(h))``, no biases.  gate and up are one stacked product."""
+
+from __future__ import annotations
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import FEED_FORWARDS, FeedForward, TensorSpec
+from tokasaurus_amd.parts.linear import Linear, Placer
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, names: dict[str, str]):
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate_up = Linear(hidden_size, [names["gate"], names["up"]], [intermediate_size] * 2)
+        self.down = Linear(intermediate_size, [names["down"]], [hidden_size])
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return self.gate_up.tensor_specs() + self.down.tensor_specs()
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        self.gate_up.load(tensors, placer)
+        self.down.load(tensors, placer)
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        prod = ops.swiglu(self.gate_up(h))
+        return self.down(prod, residual=residual)

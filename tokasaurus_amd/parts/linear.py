@@ -1,0 +1,65 @@
+"""A bias-free linear map ``y = x W^T`` (+ residual), the product every
+projection of the model goes through (``nn.Linear`` at
+tokasaurus/model/llama.py:130-149,303-315,439).  Several checkpoint tensors may
+be stacked along the output rows into one product (q|k|v, gate|up).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.parts.base import MATRIX, TensorSpec
+
+
+class Placer:
+    """Puts host tensors on the device once per (names, layout): tied tensors
+    and shared tables end up in one buffer."""
+
+    def __init__(self, dtype: torch.dtype, device: torch.device):
+        self.dtype = dtype
+        self.device = device
+        self._placed: dict[tuple, torch.Tensor] = {}
+
+    def place(self, key: tuple, make) -> torch.Tensor:
+        if key not in self._placed:
+            self._placed[key] = make()
+        return self._placed[key]
+
+    def bytes_placed(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._placed.values())
+
+
+class Linear:
+    def __init__(self, in_features: int, names: list[str], out_features: list[int]):
+        assert len(names) == len(out_features)
+        self.in_features = in_features
+        self.names = list(names)
+        self.out_features = list(out_features)
+        self.total_out = sum(out_features)
+        self.weight: torch.Tensor | None = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [TensorSpec(n, (o, self.in_features), MATRIX) for n, o in zip(self.names, self.out_features)]
+
+    def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        def make() -> torch.Tensor:
+            parts = [tensors[n] for n in self.names]
+            w = parts[0] if len(parts) == 1 else torch.cat(parts, dim=0)
+            return w.to(dtype=placer.dtype).contiguous().to(placer.device)
+
+        self.weight = placer.place(("row_major", *self.names), make)
+
+    def __call__(
+        self,
+        x: torch.Tensor,
+        residual: torch.Tensor | None = None,
+        out_f32: bool = False,
+        rows: int | None = None,
+    ) -> torch.Tensor:
+        """x [M, in] -> [M, out]; ``rows`` limits the product to the first output rows
+        of the stacked weight (a mixer that only needs its queries)."""
+        w = self.weight
+        if rows is not None and rows != self.total_out:
+            w = w[:rows]
+        return ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)

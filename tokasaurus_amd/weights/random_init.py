@@ -1,0 +1,64 @@
+"""Random weights: writes a model folder (config.json, model.safetensors) from a
+configuration and a seed.  The reference has no such mode (it only fabricates
+inputs, tokasaurus/manager/input_building.py:14-100).
+
+Every matrix is drawn from N(0, 0.02) and every norm weight from 1 + N(0, 0.01),
+in 32-bit on the host, in the sorted order of the tensor names, from one
+generator seeded with ``seed``; integer tables are drawn uniformly.  Tensors are
+stored in bfloat16, so the 32-bit engine, the bfloat16 engine and any plain
+implementation read exactly the same values.  A tied head is not drawn.
+"""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+from typing import Any
+
+import torch
+from safetensors.torch import save_file
+
+from tokasaurus_amd.models.registry import architecture_of
+from tokasaurus_amd.parts.base import INT_TABLE, MATRIX, NORM_WEIGHT, TensorSpec
+
+MATRIX_STD = 0.02
+NORM_STD = 0.01
+
+
+def draw_tensors(specs: list[TensorSpec], seed: int, store_dtype: torch.dtype = torch.bfloat16) -> dict[str, torch.Tensor]:
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(seed))
+    out: dict[str, torch.Tensor] = {}
+    for spec in sorted(specs, key=lambda s: s.name):
+        if spec.kind == MATRIX:
+            t = torch.randn(spec.shape, generator=gen, dtype=torch.float32) * MATRIX_STD
+        elif spec.kind == NORM_WEIGHT:
+            t = 1.0 + torch.randn(spec.shape, generator=gen, dtype=torch.float32) * NORM_STD
+        elif spec.kind == INT_TABLE:
+            out[spec.name] = torch.randint(0, 1 << 15, spec.shape, generator=gen, dtype=torch.int32)
+            continue
+        else:
+            raise ValueError(f"tensor {spec.name}: unknown kind {spec.kind!r}")
+        out[spec.name] = t.to(store_dtype)
+    return out
+
+
+def write_random_model(
+    folder: str | Path,
+    config: dict[str, Any],
+    seed: int,
+    store_dtype: torch.dtype = torch.bfloat16,
+) -> Path:
+    """Write ``config.json`` and ``model.safetensors`` for the architecture that
+    ``config['model_type']`` names; returns the folder."""
+    from tokasaurus_amd.models.registry import build_model
+
+    folder = Path(folder)
+    folder.mkdir(parents=True, exist_ok=True)
+    arch = architecture_of(config)
+    cfg = arch.config_from_dict(config)
+    model = build_model(arch, cfg)
+    tensors = draw_tensors(model.tensor_specs(), seed, store_dtype)
+    (folder / "config.json").write_text(json.dumps(config, indent=2) + "\n")
+    save_file({k: v.contiguous() for k, v in tensors.items()}, str(folder / "model.safetensors"))
+    return folder
