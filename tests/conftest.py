@@ -22,3 +22,6 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+from gpu_common import folders  # noqa: E402,F401  (session fixture: tiny model folders)

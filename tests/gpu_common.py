@@ -1,0 +1,22 @@
+"""Shared by the GPU tests: model folders made once per session, tolerances."""
+
+from __future__ import annotations
+
+import pytest
+
+from tiny_models import TINY, make_folder
+
+# Logits of the tiny models are of order 1.  In 32-bit the engine and the plain
+# implementation differ by the order of summation only.  In bfloat16 every
+# activation is rounded to 8 bits of mantissa on its way through two or three
+# blocks, which moves logits by about a percent of their scale.
+TOL = {
+    "float32": dict(atol=5e-5, rtol=1e-4),
+    "bfloat16": dict(atol=6e-2, rtol=5e-2),
+}
+
+
+@pytest.fixture(scope="session")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: make_folder(root / name, cfg, seed=11 + i) for i, (name, (cfg, _)) in enumerate(sorted(TINY.items()))}

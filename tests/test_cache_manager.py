@@ -1,0 +1,162 @@
+"""The cache manager: pages, block tables, groups, windows, slots."""
+
+import math
+import random
+
+import pytest
+
+from tokasaurus_amd.cache import RELEASED, CacheGroup, CacheManager, NoSpaceException, PagePool, SlotAllocator, plan_groups
+from tokasaurus_amd.parts.base import CacheNeed
+
+FULL = CacheNeed(2, 16, 0)
+
+
+def one_group(num_pages=8, page_size=4, slots=8):
+    return CacheManager([CacheGroup(FULL, (0, 1))], num_pages, page_size, slots)
+
+
+def test_reference_vectors_basic_allocation():
+    # the reference's tests/test_block_allocator.py:16-38: page 4, 8 blocks
+    m = one_group()
+    m.admit("seq1"); m.reserve("seq1", 16)
+    m.admit("seq2"); m.reserve("seq2", 9)
+    assert len(m.requests["seq1"].tables[0]) == math.ceil(16 / 4)
+    assert len(m.requests["seq2"].tables[0]) == math.ceil(9 / 4)
+    m.admit("seq3")
+    with pytest.raises(NoSpaceException):
+        m.reserve("seq3", 8)
+    assert m.requests["seq3"].tables[0] == []  # nothing was taken
+    m.check()
+
+
+def test_reference_vectors_free_and_reuse():
+    # tests/test_block_allocator.py:84-118: three 31+1-token requests take all 8 blocks in turn
+    m = one_group()
+    for name in ("a", "b", "c"):
+        m.admit(name)
+        m.reserve(name, 31)
+        m.reserve(name, 32)
+        assert sorted(m.requests[name].tables[0]) == list(range(8))
+        m.admit("other")
+        with pytest.raises(ValueError):  # NoSpaceException is a ValueError (:97-98)
+            m.reserve("other", 1)
+        m.release("other")
+        m.release(name)
+        m.check()
+    assert m.num_free_pages() == [8]
+
+
+def test_token_to_page_arithmetic_and_growth():
+    m = one_group(num_pages=16)
+    m.admit("r")
+    m.reserve("r", 4)  # exactly one page
+    assert len(m.requests["r"].tables[0]) == 1
+    m.advance("r", 4)
+    m.reserve("r", 5)  # the next token starts a page
+    assert len(m.requests["r"].tables[0]) == 2
+    m.reserve("r", 8)
+    assert len(m.requests["r"].tables[0]) == 2
+    assert m.pages_needed("r", 9) == [1] and m.pages_needed(None, 9) == [3]
+    with pytest.raises(ValueError):
+        m.advance("r", 9)  # more tokens than there is room for
+
+
+def test_lifo_reuse_is_deterministic():
+    m = one_group(num_pages=6)
+    m.admit("a"); m.reserve("a", 8)  # pages 0, 1
+    m.admit("b"); m.reserve("b", 4)  # page 2
+    assert m.requests["a"].tables[0] == [0, 1] and m.requests["b"].tables[0] == [2]
+    m.release("a")
+    m.admit("c"); m.reserve("c", 12)
+    assert m.requests["c"].tables[0] == [1, 0, 3]  # last freed first
+
+
+def test_double_free_and_unknown_pages_are_errors():
+    p = PagePool(4)
+    got = p.allocate(2)
+    p.free(got)
+    with pytest.raises(ValueError, match="twice"):
+        p.free(got)
+    with pytest.raises(ValueError):
+        p.free([99])
+    s = SlotAllocator(2)
+    a = s.allocate(); s.allocate()
+    with pytest.raises(NoSpaceException):
+        s.allocate()
+    s.free(a)
+    with pytest.raises(ValueError):
+        s.free(a)
+    m = one_group()
+    m.admit("x")
+    with pytest.raises(ValueError, match="already live"):
+        m.admit("x")
+
+
+def test_groups_by_need_and_cache_sharing():
+    win = CacheNeed(2, 16, 8)
+    needs = [FULL, win, None, FULL, win, FULL]
+    groups, where = plan_groups(needs, [None, None, None, None, None, 0])
+    assert [(g.need, g.entries) for g in groups] == [(FULL, (0, 3)), (win, (1, 4))]
+    assert where == [(0, 0), (1, 0), None, (0, 1), (1, 1), (0, 0)]  # entry 5 reads entry 0's cache
+    with pytest.raises(ValueError, match="head layout"):
+        plan_groups([FULL, CacheNeed(1, 16, 0)], [None, 0])
+    with pytest.raises(ValueError, match="further back"):
+        plan_groups([win, FULL], [None, 0])
+
+
+def test_window_pages_are_given_back_once_passed():
+    P, W = 4, 6
+    m = CacheManager([CacheGroup(FULL, (0,)), CacheGroup(CacheNeed(2, 16, W), (1,))], 16, P, 4)
+    m.admit("r")
+    n = 0
+    for step in (5, 3, 1, 1, 1, 9, 1, 1):
+        n += step
+        m.reserve("r", n)
+        # pages that this step's queries (positions n-step .. n-1) read are still held
+        first_read = max(0, (n - step) - W + 1) // P
+        assert all(p != RELEASED for p in m.requests["r"].tables[1][first_read:])
+        m.advance("r", n)
+        full, windowed = m.requests["r"].tables
+        assert all(p != RELEASED for p in full)
+        first_needed = max(0, n - W + 1) // P  # the next query sits at position n
+        assert [p == RELEASED for p in windowed] == [b < first_needed for b in range(len(windowed))]
+        m.check()
+    assert m.num_free_pages()[1] > m.num_free_pages()[0]
+    m.release("r")
+    assert m.num_free_pages() == [16, 16]
+    m.check()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_lose_no_page(seed):
+    rng = random.Random(seed)
+    P = rng.choice([1, 4, 8])
+    groups = [CacheGroup(FULL, (0, 2)), CacheGroup(CacheNeed(2, 16, rng.choice([3, 10, 40])), (1,))]
+    pages = rng.choice([6, 12, 40])
+    m = CacheManager(groups, pages, P, max_slots=5)
+    live: dict[str, int] = {}
+    counter = 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.25 and len(live) < 5:
+            name = f"r{counter}"; counter += 1
+            m.admit(name); live[name] = 0
+        elif action < 0.8 and live:
+            name = rng.choice(sorted(live))
+            new_len = live[name] + rng.choice([1, 1, 1, 2, 7, 19])
+            free_before = m.num_free_pages()
+            tables_before = [list(t) for t in m.requests[name].tables]
+            try:
+                m.reserve(name, new_len)
+            except NoSpaceException:
+                assert m.num_free_pages() == free_before and m.requests[name].tables == tables_before
+            else:
+                m.advance(name, new_len); live[name] = new_len
+        elif live:
+            name = rng.choice(sorted(live))
+            m.release(name); del live[name]
+        m.check()
+    for name in list(live):
+        m.release(name)
+    m.check()
+    assert m.num_free_pages() == [pages, pages] and m.slots.num_free == 5

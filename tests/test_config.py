@@ -1,0 +1,115 @@
+"""Configuration: config.json keys, the architecture registry, the key=value grammar."""
+
+import json
+
+import pytest
+
+from tiny_models import CONFIG_A, CONFIG_B
+from tokasaurus_amd.config import ConfigError, EngineConfig, LlamaConfig, OptionError, apply_overrides
+from tokasaurus_amd.engine.entry import RunConfig
+from tokasaurus_amd.models import ARCHITECTURES, architecture_of, build_model, config_from_folder
+
+
+def test_llama_config_reads_its_keys():
+    cfg = LlamaConfig.from_dict(CONFIG_B)
+    assert (cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads) == (96, 3, 1)
+    assert cfg.head_dim == 32  # hidden_size // num_attention_heads, llama.py:158-159
+    assert cfg.rope_scaling.rope_type == "llama3" and cfg.rope_scaling.original_max_position_embeddings == 64
+    assert cfg.rms_norm_eps == 1e-6 and not cfg.tie_word_embeddings
+    a = LlamaConfig.from_dict(CONFIG_A)
+    assert a.rope_scaling is None and a.tie_word_embeddings
+    assert LlamaConfig.from_dict(a.to_dict()) == a
+
+
+def test_missing_keys_are_named():
+    d = dict(CONFIG_A)
+    del d["rms_norm_eps"], d["rope_theta"]
+    with pytest.raises(ConfigError, match=r"rms_norm_eps.*rope_theta|rope_theta.*rms_norm_eps"):
+        LlamaConfig.from_dict(d)
+
+
+def test_kv_heads_default_and_validation():
+    d = dict(CONFIG_A)
+    del d["num_key_value_heads"]
+    assert LlamaConfig.from_dict(d).num_key_value_heads == 4
+    with pytest.raises(ConfigError, match="not a multiple"):
+        LlamaConfig.from_dict(dict(CONFIG_A, num_key_value_heads=3))
+    with pytest.raises(ConfigError, match="not divisible"):
+        LlamaConfig.from_dict(dict(CONFIG_A, hidden_size=66))
+    with pytest.raises(ConfigError, match="rope_type"):
+        LlamaConfig.from_dict(dict(CONFIG_A, rope_scaling={"rope_type": "yarn", "factor": 2.0}))
+    with pytest.raises(ConfigError, match="lacks"):
+        LlamaConfig.from_dict(dict(CONFIG_A, rope_scaling={"rope_type": "llama3", "factor": 2.0}))
+
+
+def test_eos_ids_int_or_list(tmp_path):
+    assert LlamaConfig.from_dict(dict(CONFIG_A, eos_token_id=7)).eos_token_ids == (7,)
+    assert LlamaConfig.from_dict(dict(CONFIG_A, eos_token_id=[7, 9])).eos_token_ids == (7, 9)
+    (tmp_path / "config.json").write_text(json.dumps(CONFIG_A))
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [3, 4]}))
+    _, cfg = config_from_folder(tmp_path)
+    assert cfg.eos_token_ids == (3, 4)
+
+
+def test_registry_picks_by_model_type_and_lists_known_names():
+    assert "llama" in ARCHITECTURES
+    assert architecture_of(CONFIG_A).name == "llama"
+    with pytest.raises(ConfigError, match="llama"):
+        architecture_of({"model_type": "mamba"})
+    with pytest.raises(ConfigError, match="model_type"):
+        architecture_of({})
+
+
+def test_model_is_built_from_the_config_alone():
+    for cfgd in (CONFIG_A, CONFIG_B):
+        arch = architecture_of(cfgd)
+        cfg = arch.config_from_dict(cfgd)
+        model = build_model(arch, cfg)
+        shapes = {s.name: s.shape for s in model.tensor_specs()}
+        d = cfg.head_dim
+        assert shapes["model.layers.0.self_attn.k_proj.weight"] == (cfg.num_key_value_heads * d, cfg.hidden_size)
+        assert shapes["model.layers.0.mlp.down_proj.weight"] == (cfg.hidden_size, cfg.intermediate_size)
+        assert ("lm_head.weight" in shapes) == (not cfg.tie_word_embeddings)
+        assert len(model.spec.run_order) == cfg.num_hidden_layers
+        need = model.cache_needs()[0]
+        assert (need.num_kv_heads, need.head_dim, need.window) == (cfg.num_key_value_heads, d, 0)
+
+
+def test_rope_scaling_override(tmp_path):
+    (tmp_path / "config.json").write_text(json.dumps(CONFIG_B))
+    ec = apply_overrides(EngineConfig(), ["rope_scaling=" + json.dumps({"rope_type": "linear", "factor": 2.0})])
+    _, cfg = config_from_folder(tmp_path, ec.rope_scaling_override())
+    assert cfg.rope_scaling.rope_type == "linear" and cfg.rope_scaling.factor == 2.0
+    ec = apply_overrides(EngineConfig(), ['rope_scaling={"rope_type": "default"}'])
+    _, cfg = config_from_folder(tmp_path, ec.rope_scaling_override())
+    assert cfg.rope_scaling.rope_type == "default"
+    assert EngineConfig().rope_scaling_override() == (False, None)
+
+
+def test_key_value_grammar():
+    c = apply_overrides(RunConfig(), [
+        "model=/some/dir", "kv_cache_num_tokens=(512*1024)", "page_size=8", "greedy_prefill=F",
+        "allocator_sanity_checks=T", "max_num_tokens_per_request=None", "temperature=0.7",
+        "prompt_ids=([[1, 2], [3]])", ".eager",
+    ])
+    assert c.model == "/some/dir" and c.kv_cache_num_tokens == 512 * 1024 and c.page_size == 8
+    assert c.greedy_prefill is False and c.allocator_sanity_checks is True
+    assert c.max_num_tokens_per_request is None and c.temperature == 0.7
+    assert c.prompt_ids == [[1, 2], [3]] and c.use_hipgraphs is False
+    assert apply_overrides(EngineConfig(), [".fp32"]).dtype == "float32"
+    for bad, msg in (("pagesize=4", "unknown option"), ("page_size=four", "integer"), (".nothing", "unknown method"),
+                     ("page_size", "neither"), ("greedy_prefill=maybe", "T or F"),
+                     ("kv_cache_num_tokens=(__import__('os'))", "literals")):
+        with pytest.raises(OptionError, match=msg):
+            apply_overrides(EngineConfig(), [bad])
+
+
+def test_finalize_derives_and_checks():
+    c = EngineConfig(kv_cache_num_tokens=4096, page_size=16).finalize(max_position_embeddings=131072)
+    assert c.max_num_tokens_per_request == 4096  # min(max positions, cache), common_types.py:162-166
+    assert c.kv_cache_num_blocks() == 256
+    assert EngineConfig(kv_cache_num_tokens=1 << 20).finalize(8192).max_num_tokens_per_request == 8192
+    with pytest.raises(OptionError, match="multiple"):
+        EngineConfig(kv_cache_num_tokens=100, page_size=16).finalize()
+    with pytest.raises(OptionError, match="dtype"):
+        EngineConfig(dtype="float16").finalize()

@@ -1,0 +1,223 @@
+"""Replays the same requests in every way of cutting and batching, in 32-bit and
+in bfloat16, and compares every logit row with the plain implementation."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+from gpu_common import TOL
+from replay_helpers import compare, plain_rows, portions, run_steps, tail_one_by_one, whole
+from tiny_models import TINY, random_tokens
+from tokasaurus_amd.cache import NoSpaceException
+from tokasaurus_amd.engine.batch import StepEntry
+from tokasaurus_amd.engine.runner import ModelRunner
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"A": [5, 17, 33, 97], "B": [1, 9, 70, 130], "C": [40, 150]}
+
+
+def requests_for(name):
+    cfg, _ = TINY[name]
+    return {f"r{n}": random_tokens(n, cfg["vocab_size"], 100 + n) for n in LENGTHS[name]}
+
+
+def runner_for(folders, name, dtype, tokens=512):
+    _, page = TINY[name]
+    return ModelRunner.from_folder(folders[name], dtype, page_size=page, num_pages=tokens // page, max_slots=4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_each_request_alone_and_whole(folders, name, dtype):
+    reqs = requests_for(name)
+    ref = plain_rows(folders[name], reqs)
+    runner = runner_for(folders, name, dtype)
+    for rid, toks in reqs.items():
+        got = run_steps(runner, whole(rid, toks))
+        assert len(got) == len(toks)
+        compare(got, ref, **TOL[dtype])
+    assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_32_tokens_one_by_one(folders, name, dtype):
+    reqs = {k: v for k, v in requests_for(name).items() if len(v) > 32}
+    ref = plain_rows(folders[name], reqs)
+    runner = runner_for(folders, name, dtype)
+    for rid, toks in reqs.items():
+        got = run_steps(runner, tail_one_by_one(rid, toks, 32))
+        assert len(got) == len(toks)
+        compare(got, ref, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(folders, name, dtype):
+    reqs = requests_for(name)
+    ref = plain_rows(folders[name], reqs)
+    runner = runner_for(folders, name, dtype)
+    for k, (rid, toks) in enumerate(reqs.items()):
+        sizes = [[16, 7, 2, 5, 3], [2, 2, 31, 1, 4, 9], [3, 64, 2]][k % 3]
+        got = run_steps(runner, portions(rid, toks, sizes))
+        compare(got, ref, **TOL[dtype])
+
+
+def mixed_trace(reqs: dict[str, list[int]], seed: int, max_live: int = 4):
+    """Up to four live requests; portions of some beside single tokens of others; a
+    request may sit out a step; finished requests' pages go to later ones."""
+    rng = np.random.default_rng(seed)
+    waiting = list(reqs)
+    live: dict[str, int] = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
+            live[waiting.pop(0)] = 0
+        entries, ended = [], []
+        for rid in list(live):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue  # left out of this step
+            at, toks = live[rid], reqs[rid]
+            left = len(toks) - at
+            n = 1 if (left <= 12 or rng.random() < 0.4) else int(rng.choice([2, 3, 5, 8, 13, 21]))
+            n = min(n, left)
+            entries.append((rid, toks[at:at + n], list(range(n))))
+            live[rid] = at + n
+            if live[rid] == len(toks):
+                ended.append(rid)
+                del live[rid]
+        if entries:
+            steps.append({"entries": entries, "end": ended})
+    return steps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_pages_used_again(folders, name, dtype):
+    cfg, page = TINY[name]
+    lengths = {"A": [33, 50, 21, 60, 44, 9, 38], "B": [70, 9, 130, 1, 55, 64, 90], "C": [80, 150, 33, 100, 17]}[name]
+    reqs = {f"m{i}": random_tokens(n, cfg["vocab_size"], 500 + i) for i, n in enumerate(lengths)}
+    ref = plain_rows(folders[name], reqs)
+    # room for the four longest at once, each rounded up to 64 tokens: far fewer pages than the sum
+    tokens = sum(sorted(-(-n // 64) * 64 for n in lengths)[-4:])
+    runner = runner_for(folders, name, dtype, tokens=tokens)
+    steps = mixed_trace(reqs, seed=3)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    assert any(len(t) > 1 for s in steps for _, t, _ in s["entries"] if any(len(u) == 1 for _, u, _ in s["entries"]))
+    seen_pages = set()
+    reused = False
+    orig_reserve = runner.manager.reserve
+
+    def watching_reserve(rid, n):
+        nonlocal reused
+        before = set(runner.manager.requests[rid].tables[0])
+        orig_reserve(rid, n)
+        new = set(runner.manager.requests[rid].tables[0]) - before
+        reused = reused or bool(new & seen_pages)
+        seen_pages.update(new)
+
+    runner.manager.reserve = watching_reserve
+    got = run_steps(runner, steps)
+    assert reused, "the pool was so large that no page was used twice"
+    assert len(got) == sum(lengths)
+    compare(got, ref, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_and_first_tokens(folders, dtype):
+    # prompt of 3, then 200 tokens one by one (crosses many pages, positions far beyond
+    # the rotary scaling's original length of config B)
+    cfg, _ = TINY["B"]
+    toks = random_tokens(203, cfg["vocab_size"], 77)
+    ref = plain_rows(folders["B"], {"long": toks})
+    runner = runner_for(folders, "B", dtype)
+    got = run_steps(runner, tail_one_by_one("long", toks, 200))
+    compare(got, ref, **TOL[dtype])
+    # the first tokens of a sequence, alone: 1, 2 and 3 tokens
+    for n in (1, 2, 3):
+        got = run_steps(runner, whole("long", toks[:n]))
+        compare(got, ref, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_cuttings_agree_with_each_other_closely(folders, dtype):
+    # whatever the distance to the plain implementation, two ways of cutting the same
+    # request must agree to rounding of the last accumulation
+    cfg, _ = TINY["C"]
+    toks = random_tokens(120, cfg["vocab_size"], 5)
+    runner = runner_for(folders, "C", dtype)
+    a = run_steps(runner, whole("x", toks))
+    b = run_steps(runner, portions("x", toks, [7, 2, 30, 1]))
+    c = run_steps(runner, tail_one_by_one("x", toks, 32))
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=3e-2, rtol=3e-2)
+    for other in (b, c):
+        for key, row in a.items():
+            assert torch.allclose(other[key], row, **tol), key
+
+
+def test_wanted_subset_and_empty_want(folders):
+    cfg, _ = TINY["A"]
+    toks = random_tokens(30, cfg["vocab_size"], 9)
+    ref = plain_rows(folders["A"], {"s": toks})
+    runner = runner_for(folders, "A", "float32")
+    got = run_steps(runner, [
+        {"entries": [("s", toks[:20], [])]},  # a portion nobody wants logits of
+        {"entries": [("s", toks[20:], [9, 0, 4])], "end": ["s"]},  # out of order
+    ])
+    assert sorted(p for _, p in got) == [20, 24, 29]
+    compare(got, ref, **TOL["float32"])
+    logits = runner.step([StepEntry("e", toks[:4], [])])
+    assert tuple(logits.shape) == (0, cfg["vocab_size"])
+
+
+def test_no_space_leaves_the_cache_usable(folders):
+    cfg, page = TINY["A"]
+    runner = ModelRunner.from_folder(folders["A"], "float32", page_size=page, num_pages=8, max_slots=4)
+    toks = random_tokens(40, cfg["vocab_size"], 2)
+    ref = plain_rows(folders["A"], {"a": toks})
+    got = run_steps(runner, [{"entries": [("a", toks[:20], list(range(20)))]}])
+    with pytest.raises(NoSpaceException):
+        runner.step([StepEntry("b", toks[:16], [0])])
+    runner.release("b")
+    runner.manager.check()
+    got.update({("a", 20 + k): v for (_, k), v in run_steps(runner, [{"entries": [("a", toks[20:30], list(range(10)))]}]).items()})
+    compare(got, ref, **TOL["float32"])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_program(folders, tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done' lines out."""
+    cfg, page = TINY["B"]
+    reqs = {"a": random_tokens(70, cfg["vocab_size"], 1), "b": random_tokens(41, cfg["vocab_size"], 2)}
+    ref = plain_rows(folders["B"], reqs)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": reqs["a"][:50], "want": [0, 49]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": reqs["b"][:40], "want": []},
+                                {"id": "a", "tokens": reqs["a"][50:52], "want": [0, 1]}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": reqs["a"][52:53], "want": [0]},
+                                {"id": "b", "tokens": reqs["b"][40:41], "want": [0]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": reqs["a"][53:], "want": [16]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(folders["B"]), "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "128", "--page-size", str(page)],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"]
+    V = cfg["vocab_size"]
+    expect = {0: [("a", 0), ("a", 49)], 1: [("a", 50), ("a", 51)], 2: [("a", 52), ("b", 40)], 3: [("a", 69)]}
+    for step, rows in expect.items():
+        arr = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, V)
+        assert arr.shape[0] == len(rows)
+        got = {key: torch.from_numpy(arr[i].copy()) for i, key in enumerate(rows)}
+        compare(got, ref, **TOL[dtype])

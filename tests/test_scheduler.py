@@ -1,0 +1,204 @@
+"""The scheduler's decisions, with a fake model (tokens are made up on the host)."""
+
+import math
+import random
+
+import pytest
+
+from tokasaurus_amd.cache import CacheGroup, CacheManager
+from tokasaurus_amd.engine.batch import PlannedEntry, layout
+from tokasaurus_amd.engine.scheduler import DECODING, FINISHED, PREFILLING, QUEUED, Request, Scheduler
+from tokasaurus_amd.parts.base import CacheNeed
+from tokasaurus_amd.sampling import SamplingParams
+
+
+def make(num_pages=64, page_size=4, max_tokens_per_forward=32, max_seqs=8, eos=(), optimistic=False,
+         chunk=None, slots=None):
+    cache = CacheManager([CacheGroup(CacheNeed(2, 16, 0), (0,))], num_pages, page_size, slots or max_seqs)
+    s = Scheduler(cache, max_tokens_per_forward, max_seqs, max_num_tokens_per_request=10_000,
+                  eos_token_ids=eos, optimistic=optimistic, max_prefill_chunk=chunk, sanity_checks=True)
+    return s, cache
+
+
+def req(name, prompt_len, max_tokens, **kw):
+    return Request(name, list(range(1, prompt_len + 1)), SamplingParams(max_tokens=max_tokens, **kw))
+
+
+def run_step(s, token=lambda r: 100 + len(r.completion)):
+    d = s.schedule()
+    toks = [token(r) for r in d.requests_with_output()]
+    return d, s.apply(d, toks, [0.0] * len(toks))
+
+
+def test_token_budget_and_portions():
+    s, _ = make(max_tokens_per_forward=16)
+    s.submit(req("a", 10, 4)); s.submit(req("b", 10, 4)); s.submit(req("c", 3, 4))
+    d = s.schedule()
+    # whole prompts in order and at most one cut portion (scheduler.py:541-573)
+    assert [(r.id, n) for r, n in d.prefill] == [("a", 10), ("b", 6)] and d.decode == []
+    assert [r.id for r in d.requests_with_output()] == ["a"]
+    s.apply(d, [7], [0.0])
+    d = s.schedule()
+    # a decodes (1 token), the budget left is 15: rest of b, then c
+    assert [r.id for r in d.decode] == ["a"]
+    assert [(r.id, n) for r, n in d.prefill] == [("b", 4), ("c", 3)]
+    assert d.num_tokens() == 8
+    # finishing prompts come first in the output order, then decodes (manager/types.py:259-275)
+    assert [r.id for r in d.requests_with_output()] == ["b", "c", "a"]
+
+
+def test_max_prefill_chunk_cuts_down_to_small_portions():
+    s, _ = make(chunk=3)
+    s.submit(req("a", 8, 2))
+    sizes = []
+    while s.has_work():
+        d, _ = run_step(s)
+        sizes.append([n for _, n in d.prefill])
+    assert sizes[:3] == [[3], [3], [2]]
+
+
+def test_one_token_completion_finishes_in_its_prefill_step():
+    s, cache = make()
+    s.submit(req("a", 5, 1))
+    d, done = run_step(s)
+    assert [r.id for r in done] == ["a"] and done[0].finish_reason == "length" and done[0].completion == [100]
+    assert not s.has_work() and cache.num_free_pages() == [64] and cache.slots.num_free == 8
+
+
+def test_decode_positions_and_last_token_is_not_fed_back():
+    s, cache = make(page_size=4)
+    s.submit(req("a", 6, 3))
+    held = []
+    while s.has_work():
+        d, done = run_step(s)
+        if "a" in cache.requests:
+            held.append(cache.requests["a"].num_tokens)
+    # prompt 6 -> after decode steps 7, 8; the third token is never fed (prompt + max_tokens - 1 = 8)
+    assert held == [6, 7] and done[0].completion == [100, 101, 102]
+
+
+def test_eos_stops_unless_ignored():
+    s, _ = make(eos=(101,))
+    s.submit(req("a", 4, 10)); s.submit(req("b", 4, 10, ignore_eos=True))
+    finished = {}
+    while s.has_work():
+        _, done = run_step(s)
+        finished.update({r.id: r for r in done})
+    assert finished["a"].finish_reason == "stop" and finished["a"].completion == [100, 101]
+    assert finished["b"].finish_reason == "length" and len(finished["b"].completion) == 10
+
+
+def test_admission_reserves_the_whole_life_and_is_first_in_first_out():
+    # 8 pages of 4 tokens.  a needs ceil((10+7-1)/4) = 4 pages for its life, b ceil((9+8-1)/4) = 4, c 1.
+    s, cache = make(num_pages=8, page_size=4)
+    s.submit(req("a", 10, 7)); s.submit(req("b", 9, 8)); s.submit(req("c", 2, 2))
+    d = s.schedule()
+    assert [r.id for r, _ in d.prefill] == ["a", "b"]  # c does not overtake: no pages left beside the claims
+    assert list(s.queued) == ["c"]
+    assert cache.num_free_pages() == [8 - 3 - 3]  # only the prompts' pages are taken so far
+    while "a" in cache.requests or "b" in cache.requests:
+        d, _ = run_step(s)
+        assert s.num_bumps == 0
+    assert "c" not in s.queued  # admitted once the others ended
+    while s.has_work():
+        run_step(s)
+    assert cache.num_free_pages() == [8]
+
+
+def test_max_seqs_per_forward_caps_running_requests():
+    s, _ = make(max_seqs=2)
+    for i in range(4):
+        s.submit(req(f"r{i}", 3, 3))
+    d = s.schedule()
+    assert len(d.prefill) == 2 and len(s.queued) == 2
+
+
+def test_pages_run_out_newest_is_bumped_and_restarts_at_the_head():
+    # optimistic admission: only prompts must fit.  3 pages of 4: a (4 tokens, 1 page) and b (4, 1 page),
+    # both want 8 tokens -> each needs a 2nd page at its 1st decode step, a 3rd at its 5th: the pool runs dry.
+    s, cache = make(num_pages=3, page_size=4, optimistic=True)
+    s.submit(req("a", 4, 8)); s.submit(req("b", 4, 8))
+    d, _ = run_step(s)
+    assert [r.id for r, _ in d.prefill] == ["a", "b"] and cache.num_free_pages() == [1]
+    d = s.schedule()  # both decode; a gets the last page, b (newest) is bumped
+    assert s.num_bumps == 1 and [r.id for r in d.decode] == ["a"]
+    # b lost its progress, went to the head of the queue, and (its prompt fitting again) was
+    # admitted anew in the same round: it prefills from its first token beside a's decode
+    b = s.prefilling["b"]
+    assert b.state == PREFILLING and b.prompt_done == 0 and b.completion == [] and b.times_bumped == 1
+    assert [(r.id, n) for r, n in d.prefill] == [("b", 4)]
+    s.apply(d, [100, 101], [0.0, 0.0])  # b finishes its prompt again, a decodes
+    finished = {}
+    while s.has_work():
+        _, done = run_step(s)
+        finished.update({r.id: r for r in done})
+    # both complete in full; b's restart redid everything
+    assert len(finished["a"].completion) == 8 and len(finished["b"].completion) == 8
+    assert cache.num_free_pages() == [3] and cache.slots.num_free == 8
+
+
+def test_submit_refuses_what_could_never_run():
+    s, _ = make(num_pages=4, page_size=4)
+    with pytest.raises(ValueError, match="more than the whole cache"):
+        s.submit(req("big", 16, 2))
+    with pytest.raises(ValueError, match="empty"):
+        s.submit(Request("e", [], SamplingParams()))
+    s2 = Scheduler(CacheManager([CacheGroup(CacheNeed(1, 16, 0), (0,))], 64, 4, 4), 32, 4, max_num_tokens_per_request=20)
+    with pytest.raises(ValueError, match="max_num_tokens_per_request"):
+        s2.submit(req("long", 15, 6))
+    s.submit(req("ok", 4, 2))
+    with pytest.raises(ValueError, match="already in use"):
+        s.submit(req("ok", 4, 2))
+
+
+def test_abort_frees_pages():
+    s, cache = make()
+    s.submit(req("a", 9, 5)); s.submit(req("b", 3, 5))
+    run_step(s)
+    assert s.abort("a").finish_reason == "abort" and "a" not in cache.requests
+    assert s.abort("nobody") is None
+    while s.has_work():
+        run_step(s)
+    assert cache.num_free_pages() == [64]
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("optimistic", [False, True])
+def test_random_workloads_finish_with_every_page_back(seed, optimistic):
+    rng = random.Random(seed)
+    P = rng.choice([2, 4, 16])
+    s, cache = make(num_pages=rng.choice([24, 40]), page_size=P, max_tokens_per_forward=rng.choice([8, 24]),
+                    max_seqs=rng.choice([2, 4, 8]), optimistic=optimistic, eos=(3,))
+    total = cache.num_free_pages()[0]
+    want = {}
+    for i in range(12):
+        plen, mt = rng.randint(1, 20), rng.randint(1, 12)
+        if math.ceil((plen + mt - 1) / P) > total:
+            continue
+        s.submit(req(f"r{i}", plen, mt)); want[f"r{i}"] = mt
+    finished, steps = {}, 0
+    while s.has_work():
+        d = s.schedule()
+        assert 0 < d.num_tokens() <= s.max_tokens_per_forward
+        assert len(s.prefilling) + len(s.decoding) <= s.max_seqs_per_forward
+        # the layout of the step is consistent with the cache's tables
+        planned = [PlannedEntry(r.id, r.prompt[r.prompt_done:r.prompt_done + n], [], cache.requests[r.id].slot,
+                                r.prompt_done, cache.requests[r.id].tables) for r, n in d.prefill]
+        planned += [PlannedEntry(r.id, None, [0], cache.requests[r.id].slot, r.cache_tokens(), cache.requests[r.id].tables)
+                    for r in d.decode]
+        hb = layout(planned, 10_000, 1)
+        for r_i, kv in enumerate(hb.kv_len):
+            assert math.ceil(kv / P) <= sum(1 for p in hb.block_tables[0][r_i] if p >= 0)
+        toks = [rng.choice([3, 5, 6, 7, 8, 9]) for _ in d.requests_with_output()]
+        for r in s.apply(d, toks, None):
+            finished[r.id] = r
+        steps += 1
+        assert steps < 2000
+    assert set(finished) == set(want)
+    for name, r in finished.items():
+        assert r.state == FINISHED
+        assert (r.finish_reason == "stop" and r.completion[-1] == 3) or len(r.completion) == want[name]
+    if not optimistic:
+        assert s.num_bumps == 0
+    assert cache.num_free_pages() == [total] and cache.slots.num_free == cache.slots.num_slots
+    cache.check()

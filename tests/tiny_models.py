@@ -2,15 +2,17 @@
 
 A and B differ in every size and option: head counts and grouping, sizes that are
 no power of two, number of layers, vocabulary, the norms' eps, the rotary base and
-scaling, tied or separate head, page size.  ``sharp=True`` multiplies the query and
-key projections by 10 so that attention is peaked: with the plain N(0, 0.02) weights
-scores are tiny, softmax is nearly uniform, and one missing or misplaced key among
-a hundred would disappear in the tolerance.
+scaling, tied or separate head, page size.  ``sharp=True`` scales the query and key
+projections so that scores have a standard deviation near 3 and attention is
+peaked: with the plain N(0, 0.02) weights scores are tiny, softmax is nearly
+uniform, and one missing or misplaced key among a hundred would disappear in
+the tolerance.
 """
 
 from __future__ import annotations
 
 import json
+import math
 from pathlib import Path
 
 import torch
@@ -95,7 +97,8 @@ def make_folder(folder: Path, config: dict, seed: int, sharp: bool = True) -> Pa
             for name in f.keys():
                 t = f.get_tensor(name)
                 if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
-                    t = (t.float() * 10.0).to(t.dtype)
+                    # scores ~ N(0, (sigma^2 H)^2): sigma^2 H = 3
+                    t = (t.float() * (math.sqrt(3.0 / config["hidden_size"]) / 0.02)).to(t.dtype)
                 tensors[name] = t
         save_file(tensors, str(path))
     return folder

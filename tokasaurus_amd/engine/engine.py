@@ -1,0 +1,180 @@
+"""The engine: scheduler, step function and sampler in one process.
+
+The reference spreads these over a manager process and a model worker that talk
+through queues (tokasaurus/manager/manager.py:981-1023,
+tokasaurus/model/basic_worker.py:39-173) and has no in-process generate call;
+its nearest relative is the hand-built loop of
+tokasaurus/benchmarks/bench_model.py:119-283.  Here ``Engine.generate`` takes
+token ids and returns completions; ``submit``/``step`` expose the loop.
+As in the reference, a decoded token's id stays on the GPU: the sampler writes
+it to the request's slot and the next step's embedding reads it from there
+(tokasaurus/model/basic_worker.py:101-137).
+"""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+
+import torch
+
+from tokasaurus_amd.config.engine_config import EngineConfig
+from tokasaurus_amd.engine.batch import StepEntry
+from tokasaurus_amd.engine.runner import ModelRunner
+from tokasaurus_amd.engine.scheduler import Decision, Request, Scheduler
+from tokasaurus_amd.sampling import Sampler, SamplingParams, uniform_for
+
+
+@dataclass
+class Completion:
+    request_id: str
+    prompt: list[int]
+    tokens: list[int]
+    logprobs: list[float]
+    finish_reason: str
+    times_bumped: int = 0
+
+
+@dataclass
+class Stats:
+    """The counters of the reference's stats line (tokasaurus/manager/monitoring.py:179-232)."""
+
+    steps: int = 0
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    bumps: int = 0
+    seconds: float = 0.0
+    extra: dict = field(default_factory=dict)
+
+    def as_dict(self) -> dict:
+        total = self.prefill_tokens + self.decode_tokens
+        s = max(self.seconds, 1e-9)
+        return {
+            "steps": self.steps,
+            "prefill_tokens": self.prefill_tokens,
+            "decode_tokens": self.decode_tokens,
+            "bumps": self.bumps,
+            "seconds": self.seconds,
+            "prefill_tok_per_s": self.prefill_tokens / s,
+            "decode_tok_per_s": self.decode_tokens / s,
+            "total_tok_per_s": total / s,
+            "tok_per_forward": total / max(self.steps, 1),
+            "forwards_per_s": self.steps / s,
+        }
+
+
+class Engine:
+    def __init__(self, config: EngineConfig, runner: ModelRunner | None = None):
+        if config.model is None and runner is None:
+            raise ValueError("EngineConfig.model is not set")
+        self.config = config
+        if runner is None:
+            from tokasaurus_amd.models.registry import config_from_folder
+
+            _, model_cfg = config_from_folder(config.model, config.rope_scaling_override())
+            config.finalize(getattr(model_cfg, "max_position_embeddings", None))
+            runner = ModelRunner.from_folder(
+                config.model,
+                config.dtype,
+                page_size=config.page_size,
+                num_pages=config.kv_cache_num_blocks(),
+                max_slots=config.max_seqs_per_forward,
+                rope_scaling_override=config.rope_scaling_override(),
+            )
+        else:
+            config.finalize(runner.max_positions)
+        self.runner = runner
+        limit = config.max_num_tokens_per_request or runner.max_positions
+        self.scheduler = Scheduler(
+            runner.manager,
+            max_tokens_per_forward=config.max_tokens_per_forward,
+            max_seqs_per_forward=config.max_seqs_per_forward,
+            max_num_tokens_per_request=min(limit, runner.max_positions),
+            eos_token_ids=runner.model.spec.eos_token_ids,
+            optimistic=config.bump_city_population_me,
+            max_prefill_chunk=config.max_prefill_chunk,
+            sanity_checks=config.allocator_sanity_checks,
+        )
+        self.sampler = Sampler(runner.model.device, want_logprobs=config.enable_chosen_logprobs)
+        self.stats = Stats()
+        self._next_id = 0
+        self._request_seed: dict[str, int] = {}
+
+    # ---- requests
+    def submit(self, prompt: list[int], params: SamplingParams | None = None, request_id: str | None = None) -> str:
+        params = params or SamplingParams()
+        if request_id is None:
+            request_id = f"req-{self._next_id}"
+        vocab = self.runner.model.spec.vocab_size
+        bad = [t for t in prompt if not 0 <= int(t) < vocab]
+        if bad:
+            raise ValueError(f"prompt holds token ids outside the vocabulary of {vocab}: {bad[:4]}")
+        self._request_seed[request_id] = params.seed if params.seed is not None else self._next_id
+        self._next_id += 1
+        self.scheduler.submit(Request(request_id, [int(t) for t in prompt], params))
+        return request_id
+
+    def abort(self, request_id: str) -> bool:
+        self._request_seed.pop(request_id, None)
+        return self.scheduler.abort(request_id) is not None
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ---- one step of the loop
+    def _entries(self, decision: Decision) -> list[StepEntry]:
+        entries = []
+        for req, n in decision.prefill:
+            ends = req.prompt_done + n == len(req.prompt)
+            entries.append(StepEntry(req.id, req.prompt[req.prompt_done : req.prompt_done + n], [n - 1] if ends else []))
+        for req in decision.decode:
+            entries.append(StepEntry(req.id, None, [0]))  # the token comes from the request's slot
+        return entries
+
+    def step(self) -> list[Completion]:
+        """Schedule, run and sample one batch; returns the requests that finished."""
+        t0 = time.perf_counter()
+        decision = self.scheduler.schedule()
+        self.stats.bumps = self.scheduler.num_bumps
+        if decision.empty():
+            if self.scheduler.queued:
+                raise RuntimeError("requests are queued but none can be admitted: the cache is too small for them")
+            return []
+        logits = self.runner.step(self._entries(decision))
+        out_reqs = decision.requests_with_output()
+        tokens: list[int] = []
+        logprobs: list[float] | None = None
+        if out_reqs:
+            temps = [r.params.temperature for r in out_reqs]
+            us = [
+                uniform_for(self.config.seed, self._request_seed[r.id], len(r.completion)) if r.params.temperature > 0 else 0.0
+                for r in out_reqs
+            ]
+            slots = [self.runner.manager.requests[r.id].slot for r in out_reqs]
+            ids, lps = self.sampler.sample(logits, temps, us, slots, self.runner.storage.last_token)
+            tokens = ids.tolist()  # the step's one device-to-host synchronisation
+            logprobs = lps.tolist() if lps is not None else None
+        finished = self.scheduler.apply(decision, tokens, logprobs)
+        self.stats.steps += 1
+        self.stats.prefill_tokens += sum(n for _, n in decision.prefill)
+        self.stats.decode_tokens += len(decision.decode)
+        self.stats.seconds += time.perf_counter() - t0
+        done = []
+        for r in finished:
+            self._request_seed.pop(r.id, None)
+            done.append(Completion(r.id, r.prompt, list(r.completion), list(r.logprobs), r.finish_reason or "", r.times_bumped))
+        return done
+
+    def run_until_done(self) -> list[Completion]:
+        done: list[Completion] = []
+        while self.has_work():
+            done.extend(self.step())
+        return done
+
+    def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams] | None = None) -> list[Completion]:
+        """Completions for every prompt, in the order of the prompts."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        ids = [self.submit(p, sp) for p, sp in zip(prompts, params)]
+        by_id = {c.request_id: c for c in self.run_until_done()}
+        return [by_id[i] for i in ids]

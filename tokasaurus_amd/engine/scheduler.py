@@ -1,0 +1,249 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token
+budget, decodes, finishes and frees.  Host-side only (no tensors).
+
+It keeps the reference's three first-in first-out queues queued -> prefilling ->
+decoding (tokasaurus/manager/types.py:150-250) and its rules:
+  * every decoding request gets exactly one token a step and the rest of
+    ``max_tokens_per_forward`` goes to prompts, in order, the last one possibly
+    cut (tokasaurus/manager/scheduler.py:541-573,598-602);
+  * the step that prefills the last prompt token already yields the first
+    completion token, and the last completion token is never fed back
+    (scheduler.py:674-682), so a request holds at most prompt + max_tokens - 1
+    tokens in the cache (tokasaurus/manager/types.py:94-104);
+  * at most ``max_seqs_per_forward`` requests run at a time (manager.py:898-899).
+
+Admission.  By default a request is admitted only when the pages for its whole
+life (prompt + max_tokens - 1 tokens) fit beside what the running requests may
+still claim, so pages never run out in flight.  With ``bump_city_population_me``
+(the reference's debug option of that name, tokasaurus/common_types.py:125)
+only the prompt has to fit; pages can then run out while decoding, and the
+reference's answer is used: the newest running request is taken out, its pages
+are freed, it loses its progress and goes back to the head of the queue
+(tokasaurus/manager/manager.py:745-813).  Pages of the whole prompt are taken at
+admission (tokasaurus/manager/allocator.py:324-384).
+"""
+
+from __future__ import annotations
+
+from collections import OrderedDict
+from dataclasses import dataclass, field
+
+from tokasaurus_amd.cache.manager import CacheManager
+from tokasaurus_amd.sampling.params import SamplingParams
+
+QUEUED, PREFILLING, DECODING, FINISHED = "queued", "prefilling", "decoding", "finished"
+
+
+@dataclass
+class Request:
+    id: str
+    prompt: list[int]
+    params: SamplingParams
+    state: str = QUEUED
+    prompt_done: int = 0  # prompt tokens already in the cache
+    completion: list[int] = field(default_factory=list)
+    logprobs: list[float] = field(default_factory=list)
+    finish_reason: str | None = None
+    times_bumped: int = 0
+
+    def max_cache_tokens(self) -> int:
+        return len(self.prompt) + self.params.max_tokens - 1
+
+    def cache_tokens(self) -> int:
+        """Tokens in the cache: the prompt part done plus every completion token fed back."""
+        return self.prompt_done + max(0, len(self.completion) - 1) if self.state == DECODING else self.prompt_done
+
+
+@dataclass
+class Decision:
+    """One step's work: (request, number of prompt tokens) portions, then decoding requests."""
+
+    prefill: list[tuple[Request, int]]
+    decode: list[Request]
+
+    def num_tokens(self) -> int:
+        return sum(n for _, n in self.prefill) + len(self.decode)
+
+    def empty(self) -> bool:
+        return not self.prefill and not self.decode
+
+    def requests_with_output(self) -> list[Request]:
+        """Requests that get a token from this step: prompts that end, then decodes
+        (the order of tokasaurus/manager/types.py:259-275)."""
+        return [r for r, n in self.prefill if r.prompt_done + n == len(r.prompt)] + list(self.decode)
+
+
+class Scheduler:
+    def __init__(
+        self,
+        cache: CacheManager,
+        max_tokens_per_forward: int,
+        max_seqs_per_forward: int,
+        max_num_tokens_per_request: int,
+        eos_token_ids: tuple[int, ...] = (),
+        optimistic: bool = False,
+        max_prefill_chunk: int | None = None,
+        sanity_checks: bool = False,
+    ):
+        self.cache = cache
+        self.max_tokens_per_forward = max_tokens_per_forward
+        self.max_seqs_per_forward = max_seqs_per_forward
+        self.max_num_tokens_per_request = max_num_tokens_per_request
+        self.eos_token_ids = set(eos_token_ids)
+        self.optimistic = optimistic
+        self.max_prefill_chunk = max_prefill_chunk
+        self.sanity_checks = sanity_checks
+        self.queued: "OrderedDict[str, Request]" = OrderedDict()
+        self.prefilling: "OrderedDict[str, Request]" = OrderedDict()
+        self.decoding: "OrderedDict[str, Request]" = OrderedDict()
+        self.num_bumps = 0
+
+    # ---- submit / abort
+    def submit(self, request: Request) -> None:
+        """Refuses a request that could not run even alone (the reference's
+        validate_length, tokasaurus/server/utils.py:249-259)."""
+        total = len(request.prompt) + request.params.max_tokens
+        if not request.prompt:
+            raise ValueError("empty prompt")
+        if total > self.max_num_tokens_per_request:
+            raise ValueError(
+                f"request {request.id!r}: prompt {len(request.prompt)} + max_tokens {request.params.max_tokens} "
+                f"exceeds max_num_tokens_per_request {self.max_num_tokens_per_request}"
+            )
+        pages = self.cache.blocks_for(request.max_cache_tokens())
+        if any(pages > pool.num_pages for pool in self.cache.pools):
+            raise ValueError(f"request {request.id!r} needs {pages} pages, more than the whole cache holds")
+        if request.id in self.queued or request.id in self.prefilling or request.id in self.decoding:
+            raise ValueError(f"request id {request.id!r} is already in use")
+        self.queued[request.id] = request
+
+    def abort(self, request_id: str) -> Request | None:
+        for q in (self.queued, self.prefilling, self.decoding):
+            if request_id in q:
+                req = q.pop(request_id)
+                if q is not self.queued:
+                    self.cache.release(req.id)
+                req.state, req.finish_reason = FINISHED, "abort"
+                return req
+        return None
+
+    def running(self) -> list[Request]:
+        """Decoding requests, then prefilling ones (manager/types.py:226-236)."""
+        return list(self.decoding.values()) + list(self.prefilling.values())
+
+    def has_work(self) -> bool:
+        return bool(self.queued or self.prefilling or self.decoding)
+
+    # ---- page arithmetic
+    def _free_pages(self) -> int:
+        return min(self.cache.num_free_pages())
+
+    def _held_blocks(self, req: Request) -> int:
+        return len(self.cache.requests[req.id].tables[0]) if self.cache.groups else 0
+
+    def _outstanding(self, req: Request) -> int:
+        """Pages a running request may still claim (manager/types.py:94-104)."""
+        return max(0, self.cache.blocks_for(req.max_cache_tokens()) - self._held_blocks(req))
+
+    # ---- one scheduling round
+    def schedule(self) -> Decision:
+        self._make_room_for_decoding()
+        self._admit()
+        decode = list(self.decoding.values())
+        budget = self.max_tokens_per_forward - len(decode)
+        prefill: list[tuple[Request, int]] = []
+        for req in self.prefilling.values():
+            if budget <= 0:
+                break
+            n = min(len(req.prompt) - req.prompt_done, budget)
+            if self.max_prefill_chunk:
+                n = min(n, self.max_prefill_chunk)
+            prefill.append((req, n))
+            budget -= n
+        if self.sanity_checks:
+            self.cache.check()
+        return Decision(prefill, decode)
+
+    def _make_room_for_decoding(self) -> None:
+        """Every decoding request needs room for one more token; when pages run
+        out the newest running requests are bumped until the rest fit."""
+        while True:
+            need = 0
+            for req in self.decoding.values():
+                need += max(self.cache.pages_needed(req.id, req.cache_tokens() + 1))
+            if need <= self._free_pages():
+                break
+            victims = self.running()
+            if len(victims) <= 1:
+                raise RuntimeError("a single request does not fit the cache; submit() should have refused it")
+            self._bump(victims[-1])
+        for req in self.decoding.values():
+            self.cache.reserve(req.id, req.cache_tokens() + 1)
+
+    def _bump(self, req: Request) -> None:
+        (self.prefilling if req.id in self.prefilling else self.decoding).pop(req.id)
+        self.cache.release(req.id)
+        req.state, req.prompt_done = QUEUED, 0
+        req.completion.clear()
+        req.logprobs.clear()
+        req.times_bumped += 1
+        self.num_bumps += 1
+        self.queued[req.id] = req
+        self.queued.move_to_end(req.id, last=False)
+
+    def _admit(self) -> None:
+        claimed = sum(self._outstanding(r) for r in self.running()) if not self.optimistic else 0
+        while self.queued:
+            if len(self.prefilling) + len(self.decoding) >= self.max_seqs_per_forward:
+                break
+            if self.cache.slots.num_free == 0:
+                break
+            req = next(iter(self.queued.values()))
+            prompt_pages = self.cache.blocks_for(len(req.prompt))
+            life_pages = self.cache.blocks_for(req.max_cache_tokens())
+            wanted = prompt_pages if self.optimistic else life_pages
+            if wanted > self._free_pages() - claimed:
+                break  # strictly first-in first-out: nobody overtakes the head
+            self.queued.pop(req.id)
+            self.cache.admit(req.id)
+            self.cache.reserve(req.id, len(req.prompt))
+            if not self.optimistic:
+                claimed += life_pages - prompt_pages
+            req.state = PREFILLING
+            self.prefilling[req.id] = req
+
+    # ---- after the step ran
+    def apply(self, decision: Decision, tokens: list[int], logprobs: list[float] | None = None) -> list[Request]:
+        """Advance every request of the decision; ``tokens`` are the sampled
+        tokens in the order of ``decision.requests_with_output()``.  Returns the
+        requests that finished; their pages and slots are free on return."""
+        out_reqs = decision.requests_with_output()
+        assert len(tokens) == len(out_reqs), (len(tokens), len(out_reqs))
+        for req, n in decision.prefill:
+            req.prompt_done += n
+            self.cache.advance(req.id, req.prompt_done)
+            if req.prompt_done == len(req.prompt):
+                self.prefilling.pop(req.id)
+                req.state = DECODING
+                self.decoding[req.id] = req
+        for req in decision.decode:
+            # the token fed in this step (the one sampled before) is now in the cache
+            self.cache.advance(req.id, req.prompt_done + len(req.completion))
+        finished = []
+        for i, req in enumerate(out_reqs):
+            req.completion.append(int(tokens[i]))
+            if logprobs is not None:
+                req.logprobs.append(float(logprobs[i]))
+            reason = None
+            if len(req.completion) >= req.params.max_tokens:
+                reason = "length"  # manager.py:201-204
+            if not req.params.ignore_eos and int(tokens[i]) in self.eos_token_ids:
+                reason = "stop"  # manager.py:205-206
+            if reason is not None:
+                self.decoding.pop(req.id)
+                self.cache.release(req.id)
+                req.state, req.finish_reason = FINISHED, reason
+                finished.append(req)
+        if self.sanity_checks:
+            self.cache.check()
+        return finished
