@@ -1,0 +1,245 @@
+"""Decode and prefill throughput of the Llama-3.2-1B shape on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the engine (schedule, run the model on one token
+per sequence from the paged cache, sample, read the tokens back).  The default
+run has the layer sizes of Llama-3.2-1B with seeded random weights, 8 sequences
+and a context of 8192 tokens: each sequence's prompt is prefilled by the engine
+so that the timed steps end at the context length.  One JSON line is printed:
+``value`` is decoded tokens a second at batch 8; ``prefill`` is one 2,048-token
+prompt; ``roofline`` prices the decode step against the bytes it must read;
+``points`` holds decode at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}  # dense MFMA peaks
+
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "num_hidden_layers": 16,
+    "hidden_size": 2048,
+    "num_attention_heads": 32,
+    "num_key_value_heads": 8,
+    "intermediate_size": 8192,
+    "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 131072,
+}
+CONTEXT = 8192
+PREFILL_TOKENS = 2048
+PAGE_SIZE = 16
+
+
+def parse() -> argparse.Namespace:
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=64)
+    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--context", type=int, default=CONTEXT)
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has (recorded in config)")
+    p.add_argument("--points", default="1,64", help="other decode batch sizes to measure, comma separated ('' for none)")
+    p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--eager", action="store_true", help="no HIP graphs")
+    return p.parse_args()
+
+
+def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int):
+    import torch
+
+    from tokasaurus_amd.engine.runner import DTYPES, ModelRunner, require_gpu
+    from tokasaurus_amd.models import architecture_of, build_model
+    from tokasaurus_amd.weights import draw_tensors
+
+    device = require_gpu()
+    arch = architecture_of(cfgd)
+    model = build_model(arch, arch.config_from_dict(cfgd))
+    tensors = draw_tensors(model.tensor_specs(), seed=0, device=device)
+    model.load(tensors, DTYPES[dtype], device)
+    del tensors
+    torch.cuda.empty_cache()
+    return ModelRunner(model, PAGE_SIZE, num_tokens // PAGE_SIZE, max_slots)
+
+
+def make_engine(runner, args, max_seqs: int):
+    from tokasaurus_amd.config import EngineConfig
+    from tokasaurus_amd.engine.engine import Engine
+
+    cfg = EngineConfig(
+        dtype=args.dtype, page_size=PAGE_SIZE, kv_cache_num_tokens=runner.manager.pools[0].num_pages * PAGE_SIZE,
+        max_tokens_per_forward=8192, max_seqs_per_forward=max_seqs, use_hipgraphs=not args.eager,
+        enable_chosen_logprobs=True,
+    )
+    return Engine(cfg, runner=runner)
+
+
+def decode_bytes(model, cfgd: dict, batch: int, ctx: int, elem: int) -> float:
+    L, nkv = len(model.spec.run_order), cfgd["num_key_value_heads"]
+    d = cfgd["hidden_size"] // cfgd["num_attention_heads"]
+    H, I, V = cfgd["hidden_size"], cfgd["intermediate_size"], cfgd["vocab_size"]
+    nq = cfgd["num_attention_heads"]
+    per_layer = (nq * d + 2 * nkv * d) * H + H * nq * d + 3 * H * I + 2 * H
+    weights = (L * per_layer + V * H + H) * elem  # the tied table is read once, by the head
+    if not cfgd["tie_word_embeddings"]:
+        pass  # an untied embedding is only gathered from: batch rows
+    kv = batch * ctx * 2 * nkv * d * elem * L
+    return float(weights + kv)
+
+
+def prefill_flops(cfgd: dict, layers: int, n: int) -> float:
+    d = cfgd["hidden_size"] // cfgd["num_attention_heads"]
+    H, I, V = cfgd["hidden_size"], cfgd["intermediate_size"], cfgd["vocab_size"]
+    nq, nkv = cfgd["num_attention_heads"], cfgd["num_key_value_heads"]
+    per_layer = (nq * d + 2 * nkv * d) * H + H * nq * d + 3 * H * I
+    gemm = 2.0 * n * layers * per_layer + 2.0 * V * H  # the head runs on one row
+    attn = layers * 4.0 * nq * d * (n * (n + 1) / 2)
+    return gemm + attn
+
+
+def time_decode(runner, args, batch: int, ctx: int, steps: int, warmup: int) -> float:
+    """Seconds per decode step at `batch` sequences whose timed steps end at `ctx` tokens."""
+    import torch
+
+    from tokasaurus_amd.sampling import SamplingParams
+
+    engine = make_engine(runner, args, max_seqs=max(batch, 1))
+    vocab = runner.model.spec.vocab_size
+    prompt_len = ctx - steps - warmup
+    g = torch.Generator().manual_seed(batch)
+    for _ in range(batch):
+        prompt = torch.randint(0, vocab, (prompt_len,), generator=g).tolist()
+        engine.submit(prompt, SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True))
+    while engine.scheduler.queued or engine.scheduler.prefilling:
+        engine.step()  # prefill, in portions under the token budget
+    assert len(engine.scheduler.decoding) == batch
+    for _ in range(warmup - 1):  # the step that ended the prefill gave the first token
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    for rid in list(engine.scheduler.decoding):
+        engine.abort(rid)
+    runner.manager.check()
+    return dt
+
+
+def time_prefill(runner, n: int, reps: int = 5) -> float:
+    import torch
+
+    from tokasaurus_amd.engine.batch import StepEntry
+
+    vocab = runner.model.spec.vocab_size
+    toks = torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(1)).tolist()
+    best = float("inf")
+    for i in range(reps + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry("prefill", toks, [n - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        runner.release("prefill")
+        if i > 0:
+            best = min(best, dt)
+    return best
+
+
+def main() -> int:
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    import torch
+
+    cfgd = dict(LLAMA_1B)
+    model_layers = cfgd["num_hidden_layers"]
+    if args.layers is not None:
+        cfgd["num_hidden_layers"] = args.layers
+    points = [int(b) for b in args.points.split(",") if b]
+    max_batch = max([args.batch] + points)
+    runner = build_runner(cfgd, args.dtype, num_tokens=max_batch * args.context, max_slots=max_batch)
+    elem = 2 if args.dtype == "bfloat16" else 4
+    key = "bf16" if args.dtype == "bfloat16" else "fp32"
+
+    dt = time_decode(runner, args, args.batch, args.context, args.steps, args.warmup)
+    value = args.batch / dt
+    nbytes = decode_bytes(runner.model, cfgd, args.batch, args.context, elem)
+    achieved = nbytes / dt / 1e9
+    out = {
+        "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape, context 8192)",
+        "value": round(value, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": key,
+        "data": "synthetic (seeded random weights and token ids)",
+        "config": {
+            "model": "llama-3.2-1b-shape",
+            "global_batch": args.batch,
+            "seq_len": args.context,
+            "parallelism": "single-gpu",
+            "layers": cfgd["num_hidden_layers"],
+            "model_layers": model_layers,
+            "hidden_size": cfgd["hidden_size"],
+            "num_attention_heads": cfgd["num_attention_heads"],
+            "num_key_value_heads": cfgd["num_key_value_heads"],
+            "head_dim": cfgd["hidden_size"] // cfgd["num_attention_heads"],
+            "intermediate_size": cfgd["intermediate_size"],
+            "vocab_size": cfgd["vocab_size"],
+            "page_size": PAGE_SIZE,
+            "tie_word_embeddings": cfgd["tie_word_embeddings"],
+            "rope_theta": cfgd["rope_theta"],
+            "rope_scaling": "llama3 factor 32 low 1 high 4 orig 8192",
+            "rms_norm_eps": cfgd["rms_norm_eps"],
+            "hip_graphs": not args.eager,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+        },
+    }
+    if not args.no_prefill:
+        pdt = time_prefill(runner, PREFILL_TOKENS)
+        flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], PREFILL_TOKENS)
+        out["prefill"] = {
+            "value": round(PREFILL_TOKENS / pdt, 1),
+            "tokens": PREFILL_TOKENS,
+            "ms": round(pdt * 1e3, 3),
+            "frac": round(flops / pdt / 1e12 / PEAK_TFLOPS[key], 4),
+        }
+    pts = {}
+    for b in points:
+        steps = max(8, min(args.steps, 32)) if b >= 32 else args.steps
+        pdt_b = time_decode(runner, args, b, args.context, steps, args.warmup)
+        pts[f"decode_b{b}"] = round(b / pdt_b, 1)
+    out["points"] = pts
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

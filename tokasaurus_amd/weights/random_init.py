@@ -25,17 +25,25 @@ MATRIX_STD = 0.02
 NORM_STD = 0.01
 
 
-def draw_tensors(specs: list[TensorSpec], seed: int, store_dtype: torch.dtype = torch.bfloat16) -> dict[str, torch.Tensor]:
-    gen = torch.Generator(device="cpu")
+def draw_tensors(
+    specs: list[TensorSpec],
+    seed: int,
+    store_dtype: torch.dtype = torch.bfloat16,
+    device: str | torch.device = "cpu",
+) -> dict[str, torch.Tensor]:
+    """Seeded tensors for every spec.  On the host (the default) the values are
+    a function of the seed alone; ``device`` draws them with that device's
+    generator instead (large benchmark models, where no folder is written)."""
+    gen = torch.Generator(device=device)
     gen.manual_seed(int(seed))
     out: dict[str, torch.Tensor] = {}
     for spec in sorted(specs, key=lambda s: s.name):
         if spec.kind == MATRIX:
-            t = torch.randn(spec.shape, generator=gen, dtype=torch.float32) * MATRIX_STD
+            t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * MATRIX_STD
         elif spec.kind == NORM_WEIGHT:
-            t = 1.0 + torch.randn(spec.shape, generator=gen, dtype=torch.float32) * NORM_STD
+            t = 1.0 + torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * NORM_STD
         elif spec.kind == INT_TABLE:
-            out[spec.name] = torch.randint(0, 1 << 15, spec.shape, generator=gen, dtype=torch.int32)
+            out[spec.name] = torch.randint(0, 1 << 15, spec.shape, generator=gen, dtype=torch.int32, device=device)
             continue
         else:
             raise ValueError(f"tensor {spec.name}: unknown kind {spec.kind!r}")
