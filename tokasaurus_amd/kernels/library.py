@@ -8,13 +8,13 @@ imported before the library so that both use the same HIP runtime.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_size_t, c_uint32, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_uint32, c_void_p
 
 import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
 from tokasaurus_amd.kernels import build as _build
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class KernelError(RuntimeError):
@@ -36,6 +36,8 @@ _SIGNATURES: dict[str, list] = {
     "tk_paged_attention_generic": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P]
     + [c_int] * 6
     + [c_float, _P],
+    "tk_gemm_skinny_bf16": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+    "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
     "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P],
 }
 

@@ -334,3 +334,61 @@ def sample(
         _stream(),
     )
     return ids, logprobs
+
+
+# --------------------------------------------------------------------------
+# bfloat16 matrix products on the matrix cores
+# --------------------------------------------------------------------------
+
+EPI_STORE, EPI_RESIDUAL, EPI_SWIGLU, EPI_F32 = 0, 1, 2, 3
+SKINNY_MAX_ROWS = 128
+
+
+def gemm_skinny_bf16(
+    a: torch.Tensor,
+    w: torch.Tensor,
+    residual: torch.Tensor | None = None,
+    out_f32: bool = False,
+    swiglu: bool = False,
+    waves_k: int = 0,
+    tiles: int = 0,
+) -> torch.Tensor:
+    """a [M <= 128, K] times w [N, K] transposed on the matrix cores, with the
+    epilogue fused: + residual, 32-bit output, or (``swiglu``: w is [gate | up]
+    stacked, 2I rows) silu(gate) * up -> [M, I]."""
+    _gpu(a, w, residual)
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.dtype == torch.bfloat16, "gemm_skinny: A must be bfloat16 [M, K]")
+    _need(w.dim() == 2 and w.is_contiguous() and w.dtype == torch.bfloat16, "gemm_skinny: W must be contiguous bfloat16 [N, K]")
+    m, k = a.shape
+    _need(w.shape[1] == k, f"gemm_skinny: A has K={k}, W has K={w.shape[1]}")
+    n = w.shape[0]
+    if swiglu:
+        _need(residual is None and not out_f32 and n % 2 == 0, "gemm_skinny: SwiGLU takes a [2I, K] weight, no residual, bfloat16 output")
+        n //= 2
+        epi = EPI_SWIGLU
+    elif residual is not None:
+        _need(not out_f32, "gemm_skinny: a residual cannot be combined with 32-bit output")
+        _need(residual.shape == (m, n) and residual.stride(1) == 1 and residual.dtype == torch.bfloat16,
+              "gemm_skinny: residual must be bfloat16 [M, N]")
+        epi = EPI_RESIDUAL
+    else:
+        epi = EPI_F32 if out_f32 else EPI_STORE
+    out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=a.device)
+    call(
+        "tk_gemm_skinny_bf16",
+        a.data_ptr(), a.stride(0), w.data_ptr(), out.data_ptr(), n,
+        residual.data_ptr() if residual is not None else None,
+        residual.stride(0) if residual is not None else 0,
+        m, n, k, epi, waves_k, tiles, _stream(),
+    )
+    return out
+
+
+def add(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """x + y, each rounded operand added in 32-bit and rounded once."""
+    _gpu(x, y)
+    _need(x.shape == y.shape and x.dtype == y.dtype and x.is_contiguous() and y.is_contiguous(),
+          "add: operands must be contiguous and alike")
+    out = torch.empty_like(x)
+    call("tk_add", dtype_code(x.dtype), x.data_ptr(), y.data_ptr(), out.data_ptr(), x.numel(), _stream())
+    return out

@@ -5,7 +5,6 @@ from __future__ import annotations
 
 import torch
 
-from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.parts.base import FEED_FORWARDS, FeedForward, TensorSpec
 from tokasaurus_amd.parts.linear import Linear, Placer
 
@@ -26,5 +25,4 @@ class SwiGLU(FeedForward):
         self.down.load(tensors, placer)
 
     def forward(self, h: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
-        prod = ops.swiglu(self.gate_up(h))
-        return self.down(prod, residual=residual)
+        return self.down(self.gate_up(h, swiglu=True), residual=residual)

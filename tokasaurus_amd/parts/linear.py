@@ -1,7 +1,14 @@
-"""A bias-free linear map ``y = x W^T`` (+ residual), the product every
+"""A bias-free linear map ``y = x W^T`` with a fused epilogue, the product every
 projection of the model goes through (``nn.Linear`` at
 tokasaurus/model/llama.py:130-149,303-315,439).  Several checkpoint tensors may
 be stacked along the output rows into one product (q|k|v, gate|up).
+
+Which kernel runs is decided by the storage type and the number of rows:
+  * float32: 32-bit multiply-adds throughout (the true 32-bit path);
+  * bfloat16, up to 128 rows (decode): the hand-written matrix-core kernel that
+    streams the weight once and fuses the epilogue;
+  * bfloat16, more rows (prefill): the library's matrix product, as in the
+    reference (its projections are library calls), followed by the epilogue kernel.
 """
 
 from __future__ import annotations
@@ -43,6 +50,12 @@ class Linear:
         return [TensorSpec(n, (o, self.in_features), MATRIX) for n, o in zip(self.names, self.out_features)]
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
+        if placer.dtype == torch.bfloat16 and self.in_features % 8:
+            raise ValueError(
+                f"{self.names[0]}: the bfloat16 kernels need an inner size that is a multiple of 8, "
+                f"got {self.in_features}; run this model with dtype=float32"
+            )
+
         def make() -> torch.Tensor:
             parts = [tensors[n] for n in self.names]
             w = parts[0] if len(parts) == 1 else torch.cat(parts, dim=0)
@@ -56,10 +69,25 @@ class Linear:
         residual: torch.Tensor | None = None,
         out_f32: bool = False,
         rows: int | None = None,
+        swiglu: bool = False,
     ) -> torch.Tensor:
-        """x [M, in] -> [M, out]; ``rows`` limits the product to the first output rows
-        of the stacked weight (a mixer that only needs its queries)."""
+        """x [M, in] -> [M, out].  ``residual``: returns residual + product (the
+        product rounded to the storage type first).  ``out_f32``: 32-bit output.
+        ``swiglu``: the weight is [gate | up]; returns silu(gate) * up.
+        ``rows`` limits the product to the first output rows of the stacked
+        weight (a mixer that only needs its queries)."""
         w = self.weight
         if rows is not None and rows != self.total_out:
             w = w[:rows]
-        return ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)
+        m = x.shape[0]
+        if w.dtype == torch.bfloat16 and m > 0:
+            if m <= ops.SKINNY_MAX_ROWS:
+                return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu)
+            prod = torch.mm(x, w.t())  # library matrix product (hipBLASLt), 32-bit accumulation
+            if swiglu:
+                return ops.swiglu(prod)
+            if residual is not None:
+                return ops.add(prod, residual.contiguous())
+            return prod.float() if out_f32 else prod
+        out = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)
+        return ops.swiglu(out) if swiglu else out
