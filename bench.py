@@ -43,6 +43,10 @@ PREFILL_TOKENS = 2048
 PAGE_SIZE = 16
 
 
+def say(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
 def parse() -> argparse.Namespace:
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -87,7 +91,7 @@ def make_engine(runner, args, max_seqs: int):
     return Engine(cfg, runner=runner)
 
 
-def decode_bytes(model, cfgd: dict, batch: int, ctx: int, elem: int) -> float:
+def decode_bytes(model, cfgd: dict, batch: int, ctx: float, elem: int) -> float:
     L, nkv = len(model.spec.run_order), cfgd["num_key_value_heads"]
     d = cfgd["hidden_size"] // cfgd["num_attention_heads"]
     H, I, V = cfgd["hidden_size"], cfgd["intermediate_size"], cfgd["vocab_size"]
@@ -118,15 +122,21 @@ def time_decode(runner, args, batch: int, ctx: int, steps: int, warmup: int) -> 
 
     engine = make_engine(runner, args, max_seqs=max(batch, 1))
     vocab = runner.model.spec.vocab_size
-    prompt_len = ctx - steps - warmup
+    # Prompts are prefilled by the engine under its token budget, so the first
+    # sequences already decode while the last are prefilled: `batch` + 8 tokens of
+    # slack keep every sequence within `ctx` when the timed steps end.
+    prompt_len = ctx - steps - warmup - batch - 8
     g = torch.Generator().manual_seed(batch)
     for _ in range(batch):
         prompt = torch.randint(0, vocab, (prompt_len,), generator=g).tolist()
-        engine.submit(prompt, SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True))
+        engine.submit(prompt, SamplingParams(temperature=0.0, max_tokens=ctx - prompt_len, ignore_eos=True))
+    t0 = time.perf_counter()
     while engine.scheduler.queued or engine.scheduler.prefilling:
         engine.step()  # prefill, in portions under the token budget
-    assert len(engine.scheduler.decoding) == batch
-    for _ in range(warmup - 1):  # the step that ended the prefill gave the first token
+    torch.cuda.synchronize()
+    say(f"batch {batch}: prefilled {batch} x {prompt_len} tokens in {time.perf_counter() - t0:.1f}s")
+    assert len(engine.scheduler.decoding) == batch, (len(engine.scheduler.decoding), batch)
+    for _ in range(warmup):
         engine.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -134,10 +144,14 @@ def time_decode(runner, args, batch: int, ctx: int, steps: int, warmup: int) -> 
         engine.step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
+    held = [rc.num_tokens for rc in runner.manager.requests.values()]
+    assert len(held) == batch and max(held) <= ctx, (len(held), max(held), ctx)
+    mean_ctx = sum(held) / len(held) - steps / 2  # mean over the timed steps
     for rid in list(engine.scheduler.decoding):
         engine.abort(rid)
     runner.manager.check()
-    return dt
+    say(f"batch {batch}: {dt * 1e3:.3f} ms a step, mean context {mean_ctx:.0f}")
+    return dt, mean_ctx
 
 
 def time_prefill(runner, n: int, reps: int = 5) -> float:
@@ -177,9 +191,9 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
 
-    dt = time_decode(runner, args, args.batch, args.context, args.steps, args.warmup)
+    dt, mean_ctx = time_decode(runner, args, args.batch, args.context, args.steps, args.warmup)
     value = args.batch / dt
-    nbytes = decode_bytes(runner.model, cfgd, args.batch, args.context, elem)
+    nbytes = decode_bytes(runner.model, cfgd, args.batch, mean_ctx, elem)
     achieved = nbytes / dt / 1e9
     out = {
         "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape, context 8192)",
@@ -224,6 +238,7 @@ def main() -> int:
     }
     if not args.no_prefill:
         pdt = time_prefill(runner, PREFILL_TOKENS)
+        say(f"prefill of {PREFILL_TOKENS} tokens: {pdt * 1e3:.2f} ms")
         flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], PREFILL_TOKENS)
         out["prefill"] = {
             "value": round(PREFILL_TOKENS / pdt, 1),
@@ -234,7 +249,7 @@ def main() -> int:
     pts = {}
     for b in points:
         steps = max(8, min(args.steps, 32)) if b >= 32 else args.steps
-        pdt_b = time_decode(runner, args, b, args.context, steps, args.warmup)
+        pdt_b, _ = time_decode(runner, args, b, args.context, steps, args.warmup)
         pts[f"decode_b{b}"] = round(b / pdt_b, 1)
     out["points"] = pts
     print(json.dumps(out))
