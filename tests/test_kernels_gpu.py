@@ -1,0 +1,81 @@
+"""Each kernel alone against a plain reference, at sizes other than the engine's."""
+
+import math
+
+import pytest
+import torch
+
+from kernel_refs import attention_reference, make_paged_case
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(t: torch.Tensor, dtype=None) -> torch.Tensor:
+    t = t.to(dtype) if dtype is not None else t
+    return t.cuda().contiguous()
+
+
+# --------------------------------------------------------------------------
+# attention
+# --------------------------------------------------------------------------
+
+ATTN_CASES = [
+    # (q_lens, kv_lens, nq, nkv, d, page, window)
+    ([1, 1, 1], [700, 33, 1], 8, 2, 64, 16, 0),  # decode, one request of a single key
+    ([37], [37], 4, 4, 32, 8, 0),  # a whole prompt, no grouping
+    ([20, 1, 5], [150, 260, 5], 6, 2, 64, 16, 0),  # a portion after a past, beside a decode and a short prompt
+    ([70, 2], [130, 64], 3, 1, 32, 8, 0),  # group of 3: rows of one token straddle tiles
+    ([16, 1], [16, 17], 4, 2, 16, 4, 0),  # exactly one tile of one page size 4; head size 16
+    ([9, 1, 40], [300, 299, 90], 8, 2, 48, 16, 0),  # head size 48: half a 32-wide step
+    ([1, 3], [1000, 515], 32, 8, 128, 16, 0),  # head size 128, many heads
+    ([33, 1, 1], [200, 200, 31], 4, 2, 64, 16, 40),  # a window: far keys must not be read
+    ([5], [77], 20, 1, 16, 4, 0),  # group of 20: more rows of one token than a tile
+]
+
+
+def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1):
+    from tokasaurus_amd.kernels import ops
+
+    dtype = torch.bfloat16 if kind != "generic_f32" else torch.float32
+    q = dev(case["q"], dtype)
+    kc, vc = dev(case["kcache"], dtype), dev(case["vcache"], dtype)
+    table = dev(case["table"])
+    if kind.startswith("generic"):
+        token_req = torch.tensor([r for r, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32).cuda()
+        positions = torch.tensor([kv - ql + j for ql, kv in zip(q_lens, kv_lens) for j in range(ql)], dtype=torch.int32).cuda()
+        return ops.paged_attention_generic(q, kc, vc, table, token_req, positions, nq, nkv, d, page, window=window)
+    tile_req, tile_row0 = ops.attention_tiles(q_lens, nq // nkv, row_tiles)
+    max_kv = max(kv_lens)
+    split = split or ops.attention_split(max_kv, len(tile_req), nkv)
+    return ops.paged_attention_mfma(
+        q, kc, vc, table, dev(case["q_start"]), dev(case["kv_len"]),
+        torch.tensor(tile_req, dtype=torch.int32).cuda(), torch.tensor(tile_row0, dtype=torch.int32).cuda(),
+        row_tiles, nq, nkv, d, page, max_kv, split, window=window,
+    )
+
+
+@pytest.mark.parametrize("case_id", range(len(ATTN_CASES)))
+@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma", "mfma_split32", "mfma_rt2"])
+def test_paged_attention(kind, case_id):
+    q_lens, kv_lens, nq, nkv, d, page, window = ATTN_CASES[case_id]
+    dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
+    case = make_paged_case(q_lens, kv_lens, nq, nkv, d, page, seed=case_id, dtype=dtype)
+    ref = attention_reference(case, q_lens, kv_lens, nq, nkv, d, window=window)
+    split = 32 if kind == "mfma_split32" else (64 if kind == "mfma_rt2" else None)
+    got = run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=split,
+                        row_tiles=2 if kind == "mfma_rt2" else 1).float().cpu()
+    assert torch.isfinite(got).all()
+    # values are of order 1; bfloat16 rounds the probabilities and the output to 8 bits
+    tol = dict(atol=2e-5, rtol=1e-4) if kind == "generic_f32" else dict(atol=2e-2, rtol=2e-2)
+    err = (got - ref).abs()
+    bad = err > tol["atol"] + tol["rtol"] * ref.abs()
+    assert not bad.any(), f"first wrong row {int(bad.any(1).nonzero()[0])}, largest error {float(err.max()):.3e}"
+
+
+def test_attention_splits_agree():
+    """The same decode with different splits: equal beyond rounding of the merge."""
+    q_lens, kv_lens, nq, nkv, d, page = [1, 1], [2000, 777], 8, 2, 64, 16
+    case = make_paged_case(q_lens, kv_lens, nq, nkv, d, page, seed=5, dtype=torch.bfloat16)
+    outs = [run_attention("mfma", case, q_lens, kv_lens, nq, nkv, d, page, 0, split=s).float() for s in (4096, 512, 128, 32)]
+    for o in outs[1:]:
+        assert torch.allclose(o, outs[0], atol=1e-2, rtol=1e-2)

@@ -1,0 +1,342 @@
+// Paged attention on the gfx950 matrix cores, bfloat16 storage, 32-bit softmax.
+// One kernel serves prompt portions and single decoded tokens.
+//
+// Rows.  For a request and a kv head, the rows are the pairs (token of this step,
+// query head of the kv head's group), numbered token * group + head.  A wavefront
+// owns RT tiles of 16 consecutive rows and walks the keys its rows may see in
+// steps of 32.  With the keys as the first operand of v_mfma_f32_16x16x32_bf16
+// and the queries as the second,
+//     S^T[key 4q+j][row r]  is element j of lane (r = lane % 16, q = lane / 16),
+// so a lane holds, for ONE row, 4 keys of each 16-key block.  These 8 numbers
+// are exactly what the lane must provide as the second operand of the product
+// O^T = V^T P^T, if slot 8q+j of that product's inner index stands for key 4q+j
+// of the first block and slot 8q+4+j for key 4q+j of the second.  The value
+// pages are stored transposed ([d][P]), so the matching first operand is read
+// with two 8-byte loads per lane.  Nothing passes through LDS.
+//
+//   K pages: [page][kv head][P][d]      V pages: [page][kv head][d][P], P % 4 == 0
+//
+// Splits.  The keys of a tile are cut at absolute multiples of `split`; each
+// (tile, kv head, split) is one wavefront.  A tile with one split writes the
+// output; otherwise partial (max, sum, weighted values) go to scratch and
+// tk_attention_merge adds them in split order.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+struct AttnArgs {
+  const bf16_t* q;
+  int q_stride;
+  bf16_t* out;
+  int out_stride;
+  const bf16_t* kcache;
+  const bf16_t* vcache;
+  const int* block_table;
+  int table_stride;
+  const int* q_start;   // [requests + 1]
+  const int* kv_len;    // [requests]
+  const int* tile_req;  // [tiles]
+  const int* tile_row0; // [tiles]
+  int n_tiles;
+  int nq, nkv, group, P, window;
+  float scale;
+  int split;       // keys per split, a multiple of 32
+  int max_splits;  // splits a tile may have (size of the scratch)
+  float* part_o;   // [tiles][nkv][max_splits][16 * RT][D]
+  float* part_ml;  // [tiles][nkv][max_splits][16 * RT][2]
+};
+
+struct TileRange {
+  int req, row0, qs, qlen, kvl, n_rows, lo, hi, s_first, s_last;
+};
+
+__device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int rows_per_tile) {
+  TileRange t;
+  t.req = a.tile_req[tile];
+  t.row0 = a.tile_row0[tile];
+  t.qs = a.q_start[t.req];
+  t.qlen = a.q_start[t.req + 1] - t.qs;
+  t.kvl = a.kv_len[t.req];
+  t.n_rows = t.qlen * a.group;
+  const int first_tok = t.row0 / a.group;
+  const int last_tok = min(t.row0 + rows_per_tile - 1, t.n_rows - 1) / a.group;
+  const int pos_first = t.kvl - t.qlen + first_tok;
+  t.hi = t.kvl - t.qlen + last_tok;
+  t.lo = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+  t.s_first = t.lo / a.split;
+  t.s_last = t.hi / a.split;
+  return t;
+}
+
+template <int DT, int RT>
+__global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
+  constexpr int D = DT * 16;
+  constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head size
+  const int lane = threadIdx.x;
+  const int r = lane & 15, q = lane >> 4;
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const TileRange t = tile_range(a, tile, 16 * RT);
+  const int s = t.s_first + blockIdx.z;
+  if (s > t.s_last) return;
+  const int nsp = t.s_last - t.s_first + 1;
+  const int k_begin = max((t.lo >> 5) << 5, s * a.split);
+  const int k_end = min(t.hi + 1, (s + 1) * a.split);
+  const int* table = a.block_table + (size_t)t.req * a.table_stride;
+  const int P = a.P;
+
+  // this lane's row in each of the RT tiles
+  int pos_r[RT], lo_r[RT];
+  bf16x8_t qv[RT][KS];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int flat = t.row0 + rt * 16 + r;
+    const bool valid = flat < t.n_rows;
+    const int fl = valid ? flat : t.n_rows - 1;
+    const int tok = fl / a.group, g = fl - tok * a.group;
+    const int pos = t.kvl - t.qlen + tok;
+    pos_r[rt] = valid ? pos : -1;
+    lo_r[rt] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    const bf16_t* qp = a.q + (size_t)(t.qs + tok) * a.q_stride + (size_t)(kvh * a.group + g) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + q * 8;
+      if (d0 < D) {
+        qv[rt][ks] = *(const bf16x8_t*)(qp + d0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[rt][ks][e] = (__bf16)0.f;
+      }
+    }
+  }
+
+  float m_run[RT], l_run[RT];
+  f32x4_t acc[RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    m_run[rt] = -INFINITY;
+    l_run[rt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int kb = k_begin; kb < k_end; kb += 32) {
+    // keys: lane (r, q) reads 8 values of key kb + 16 blk + r for every 32-wide step
+    bf16x8_t kv[2][KS];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int kk = min(max(kb + blk * 16 + r, t.lo), t.hi);
+      const int page = table[kk / P];
+      const bf16_t* kp = a.kcache + ((size_t)((size_t)page * a.nkv + kvh) * P + (kk % P)) * D;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 32 + q * 8;
+        if (d0 < D) {
+          kv[blk][ks] = *(const bf16x8_t*)(kp + d0);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) kv[blk][ks][e] = (__bf16)0.f;
+        }
+      }
+    }
+    // values: lane (r, q) reads, for d = 16 dt + r, keys kb + 16 blk + 4q .. + 3
+    bf16x8_t vv[DT];
+    {
+      const bf16_t* vp[2];
+      bool ok[2][4];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        const int k4 = kb + blk * 16 + q * 4;
+        int kc = k4;
+        if (kc > t.hi) kc = t.hi & ~3;
+        if (kc + 3 < t.lo) kc = t.lo & ~3;
+        const int page = table[kc / P];
+        vp[blk] = a.vcache + ((size_t)((size_t)page * a.nkv + kvh) * D + r) * P + (kc % P);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ok[blk][j] = (k4 + j >= t.lo) && (k4 + j <= t.hi) && kc == k4;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          const bf16x4_t x = *(const bf16x4_t*)(vp[blk] + (size_t)dt * 16 * P);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) vv[dt][blk * 4 + j] = ok[blk][j] ? x[j] : (__bf16)0.f;
+        }
+      }
+    }
+
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv[0][ks], qv[rt][ks], st[0], 0, 0, 0);
+        st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv[1][ks], qv[rt][ks], st[1], 0, 0, 0);
+      }
+      float sc[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int key = kb + blk * 16 + q * 4 + j;
+          const bool seen = key >= lo_r[rt] && key <= pos_r[rt];
+          const float v = seen ? st[blk][j] * a.scale : -INFINITY;
+          sc[blk * 4 + j] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[rt], mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __expf(m_run[rt] - m_use);  // exp(-inf) = 0 while nothing was seen
+      float psum = 0.f;
+      bf16x8_t pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __expf(sc[e] - m_use);
+        psum += p;
+        pb[e] = (__bf16)p;
+      }
+      m_run[rt] = m_new;
+      l_run[rt] = l_run[rt] * alpha + psum;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[rt][dt] *= alpha;
+        acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[dt], pb, acc[rt][dt], 0, 0, 0);
+      }
+    }
+  }
+
+  // acc[rt][dt][j] of lane (r, q) is O^T[d = 16 dt + 4q + j][row r]
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float l = l_run[rt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int flat = t.row0 + rt * 16 + r;
+    if (flat >= t.n_rows) continue;
+    if (nsp == 1) {
+      const int tok = flat / a.group, g = flat - tok * a.group;
+      bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
+      const float inv = 1.0f / l;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pk.h[j] = __float2bfloat16(acc[rt][dt][j] * inv);
+        *(uint2*)(op + dt * 16 + q * 4) = pk.u;
+      }
+    } else {
+      const size_t item = ((size_t)tile * a.nkv + kvh) * a.max_splits + (s - t.s_first);
+      float* po = a.part_o + (item * (16 * RT) + rt * 16 + r) * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(f32x4_t*)(po + dt * 16 + q * 4) = acc[rt][dt];
+      if (q == 0) {
+        float* pm = a.part_ml + (item * (16 * RT) + rt * 16 + r) * 2;
+        pm[0] = m_run[rt];
+        pm[1] = l;
+      }
+    }
+  }
+}
+
+// Adds the partial results of a tile's splits in split order.
+template <int RT>
+__global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D) {
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const TileRange t = tile_range(a, tile, 16 * RT);
+  const int nsp = t.s_last - t.s_first + 1;
+  if (nsp == 1) return;
+  const int rows = min(16 * RT, t.n_rows - t.row0);
+  const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
+  for (int i = threadIdx.x; i < rows * D; i += blockDim.x) {
+    const int row = i / D, d = i - row * D;
+    float m = -INFINITY;
+    for (int sp = 0; sp < nsp; ++sp)
+      m = fmaxf(m, a.part_ml[((item0 + sp) * (16 * RT) + row) * 2]);
+    float l = 0.f, o = 0.f;
+    for (int sp = 0; sp < nsp; ++sp) {
+      const size_t base = (item0 + sp) * (16 * RT) + row;
+      const float ms = a.part_ml[base * 2];
+      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
+      l += w * a.part_ml[base * 2 + 1];
+      o += w * a.part_o[base * D + d];
+    }
+    const int flat = t.row0 + row;
+    const int tok = flat / a.group, g = flat - tok * a.group;
+    a.out[(size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D + d] =
+        __float2bfloat16(o / l);
+  }
+}
+
+template <int DT, int RT>
+static void launch_attn(const AttnArgs& a, int grid_splits, hipStream_t stream) {
+  hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, RT>), dim3(a.n_tiles, a.nkv, grid_splits),
+                     dim3(64), 0, stream, a);
+}
+
+template <int RT>
+static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, hipStream_t stream) {
+  switch (dt) {
+    case 1: launch_attn<1, RT>(a, grid_splits, stream); return true;
+    case 2: launch_attn<2, RT>(a, grid_splits, stream); return true;
+    case 3: launch_attn<3, RT>(a, grid_splits, stream); return true;
+    case 4: launch_attn<4, RT>(a, grid_splits, stream); return true;
+    case 5: launch_attn<5, RT>(a, grid_splits, stream); return true;
+    case 6: launch_attn<6, RT>(a, grid_splits, stream); return true;
+    case 7: launch_attn<7, RT>(a, grid_splits, stream); return true;
+    case 8: launch_attn<8, RT>(a, grid_splits, stream); return true;
+    default: return false;
+  }
+}
+
+// Rows per tile are 16 * row_tiles (1 or 2).  `tile_req`/`tile_row0` list the
+// tiles; `grid_splits` is an upper bound on the splits of any tile and
+// `max_splits` the number the scratch has room for (grid_splits <= max_splits).
+// part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
+// tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when
+// max_splits is 1).  merge != 0 also launches the merge of split tiles.
+extern "C" int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
+                                       const void* kcache, const void* vcache,
+                                       const int* block_table, int table_stride,
+                                       const int* q_start, const int* kv_len,
+                                       const int* tile_req, const int* tile_row0, int n_tiles,
+                                       int row_tiles, int nq, int nkv, int d, int P, int window,
+                                       float scale, int split, int grid_splits, int max_splits,
+                                       float* part_o, float* part_ml, hipStream_t stream) {
+  TK_REQUIRE(n_tiles >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_mfma: bad sizes tiles=%d nq=%d nkv=%d", n_tiles, nq, nkv);
+  TK_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attention_mfma: head size %d is not a multiple of 16 up to 128", d);
+  TK_REQUIRE(P > 0 && P % 4 == 0, "attention_mfma: page size %d is not a multiple of 4", P);
+  TK_REQUIRE(row_tiles == 1 || row_tiles == 2, "attention_mfma: row_tiles %d outside 1..2", row_tiles);
+  TK_REQUIRE(split > 0 && split % 32 == 0, "attention_mfma: split %d is not a multiple of 32", split);
+  TK_REQUIRE(grid_splits >= 1 && grid_splits <= max_splits && grid_splits < 65536, "attention_mfma: splits %d of %d", grid_splits, max_splits);
+  TK_REQUIRE(max_splits == 1 || (part_o && part_ml), "attention_mfma: split tiles need scratch");
+  TK_REQUIRE(q_stride >= nq * d && out_stride >= nq * d && q_stride % 8 == 0 && out_stride % 4 == 0,
+             "attention_mfma: row strides %d/%d too short or unaligned", q_stride, out_stride);
+  TK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 7) == 0 && ((uintptr_t)out & 7) == 0,
+             "attention_mfma: operands must be 16-byte aligned");
+  TK_REQUIRE(nkv < 65536, "attention_mfma: too many kv heads");
+  if (n_tiles == 0) return 0;
+  AttnArgs a;
+  a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
+  a.kcache = (const bf16_t*)kcache; a.vcache = (const bf16_t*)vcache;
+  a.block_table = block_table; a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len;
+  a.tile_req = tile_req; a.tile_row0 = tile_row0; a.n_tiles = n_tiles;
+  a.nq = nq; a.nkv = nkv; a.group = nq / nkv; a.P = P; a.window = window; a.scale = scale;
+  a.split = split; a.max_splits = max_splits; a.part_o = part_o; a.part_ml = part_ml;
+  const bool ok = row_tiles == 1 ? launch_attn_d<1>(a, d / 16, grid_splits, stream)
+                                 : launch_attn_d<2>(a, d / 16, grid_splits, stream);
+  TK_REQUIRE(ok, "attention_mfma: no kernel for head size %d", d);
+  TK_CHECK_LAUNCH("paged_attention_mfma");
+  if (max_splits > 1) {
+    if (row_tiles == 1)
+      hipLaunchKernelGGL((attention_merge_kernel<1>), dim3(n_tiles, nkv), dim3(256), 0, stream, a, d);
+    else
+      hipLaunchKernelGGL((attention_merge_kernel<2>), dim3(n_tiles, nkv), dim3(256), 0, stream, a, d);
+    TK_CHECK_LAUNCH("attention_merge");
+  }
+  return 0;
+}

@@ -296,6 +296,111 @@ def paged_attention_generic(
     return out
 
 
+def attention_mfma_supports(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core attention kernel takes this storage type, head size and page size."""
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128 and page_size % 4 == 0
+
+
+def attention_tiles(q_lens: list[int], group: int, row_tiles: int) -> tuple[list[int], list[int]]:
+    """The tiles of 16 * row_tiles rows that cover every request's (token, head of the group) pairs."""
+    rows = 16 * row_tiles
+    tile_req: list[int] = []
+    tile_row0: list[int] = []
+    for r, n in enumerate(q_lens):
+        for row0 in range(0, n * group, rows):
+            tile_req.append(r)
+            tile_row0.append(row0)
+    return tile_req, tile_row0
+
+
+def attention_split(max_kv_len: int, n_tiles: int, nkv: int, target_waves: int = 4096) -> int:
+    """Keys per split (a multiple of 128) so that about ``target_waves`` wavefronts share the work."""
+    per = max_kv_len * max(n_tiles * nkv, 1) / target_waves
+    return max(128, -(-int(per) // 128) * 128)
+
+
+def paged_attention_mfma(
+    q: torch.Tensor,
+    kcache: torch.Tensor,
+    vcache: torch.Tensor,
+    block_table: torch.Tensor,
+    q_start: torch.Tensor,
+    kv_len: torch.Tensor,
+    tile_req: torch.Tensor,
+    tile_row0: torch.Tensor,
+    row_tiles: int,
+    nq: int,
+    nkv: int,
+    head_dim: int,
+    page_size: int,
+    max_kv_len: int,
+    split: int,
+    window: int = 0,
+    scale: float | None = None,
+    out: torch.Tensor | None = None,
+    scratch: tuple[torch.Tensor, torch.Tensor] | None = None,
+) -> torch.Tensor:
+    """Attention of every token of the batch over its request's pages on the
+    matrix cores (bfloat16).  ``q`` is 2-d and its first nq*d columns are the
+    query heads; request r owns tokens q_start[r]..q_start[r+1]-1, the last of
+    them at position kv_len[r]-1.  ``max_kv_len`` bounds kv_len (it sizes the
+    grid and the scratch, so it may be larger than any request's)."""
+    _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * head_dim and q.dtype == torch.bfloat16,
+          "attention_mfma: q must be bfloat16, 2-d with unit inner stride and nq*d leading columns")
+    n = q.shape[0]
+    for t, name in ((block_table, "block_table"), (q_start, "q_start"), (kv_len, "kv_len"),
+                    (tile_req, "tile_req"), (tile_row0, "tile_row0")):
+        _i32(t, name)
+    _need(block_table.dim() == 2, "block_table must be [requests, width]")
+    requests = kv_len.numel()
+    _need(q_start.numel() == requests + 1 and block_table.shape[0] >= requests,
+          "attention_mfma: q_start, kv_len and block_table disagree on the number of requests")
+    _need(block_table.shape[1] * page_size >= max_kv_len or requests == 0,
+          "attention_mfma: block table narrower than the longest request")
+    n_tiles = tile_req.numel()
+    _need(tile_row0.numel() == n_tiles, "attention_mfma: tile lists differ in length")
+    pages = kcache.shape[0]
+    _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
+          "attention_mfma: key pages must be contiguous [pages, nkv, P, d]")
+    _need(tuple(vcache.shape) == (pages, nkv, head_dim, page_size) and vcache.is_contiguous(),
+          "attention_mfma: value pages must be contiguous [pages, nkv, d, P]")
+    _need(kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16, "attention_mfma: the cache must be bfloat16")
+    _need(attention_mfma_supports(q.dtype, head_dim, page_size),
+          f"attention_mfma: head size {head_dim} / page size {page_size} not supported")
+    _need(split > 0 and split % 32 == 0, "attention_mfma: split must be a positive multiple of 32")
+    if out is None:
+        out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
+    else:
+        _need(out.shape == (n, nq * head_dim) and out.dtype == q.dtype and out.stride(1) == 1, "attention_mfma: bad out")
+    max_splits = max(1, -(-max_kv_len // split))
+    part_o = part_ml = None
+    if max_splits > 1:
+        rows = 16 * row_tiles
+        items = n_tiles * nkv * max_splits * rows
+        if scratch is not None:
+            part_o, part_ml = scratch
+            _need(part_o.dtype == torch.float32 and part_ml.dtype == torch.float32
+                  and part_o.numel() >= items * head_dim and part_ml.numel() >= items * 2,
+                  "attention_mfma: scratch too small")
+        else:
+            part_o = torch.empty((items * head_dim,), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((items * 2,), dtype=torch.float32, device=q.device)
+    call(
+        "tk_paged_attention_mfma",
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+        kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+        q_start.data_ptr(), kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(),
+        n_tiles, row_tiles, nq, nkv, head_dim, page_size, int(window),
+        float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
+        split, max_splits, max_splits,
+        part_o.data_ptr() if part_o is not None else None,
+        part_ml.data_ptr() if part_ml is not None else None,
+        _stream(),
+    )
+    return out
+
+
 def sample(
     logits: torch.Tensor,
     temperature: torch.Tensor,

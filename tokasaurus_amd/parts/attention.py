@@ -11,6 +11,7 @@ the last ``window`` of them.
 from __future__ import annotations
 
 import math
+from dataclasses import dataclass
 
 import torch
 
@@ -26,6 +27,32 @@ from tokasaurus_amd.parts.base import (
     TensorSpec,
 )
 from tokasaurus_amd.parts.linear import Linear, Placer
+
+
+@dataclass
+class AttentionPlan:
+    """How the step's rows are cut into tiles and its keys into splits; made once
+    a step for each group size and shared by the layers."""
+
+    tile_req: torch.Tensor
+    tile_row0: torch.Tensor
+    row_tiles: int
+    max_kv_len: int
+    split: int
+
+
+def attention_plan(ctx: StepContext, group: int, nkv: int) -> AttentionPlan:
+    key = ("attention_plan", group, nkv)
+    plan = ctx.extras.get(key)
+    if plan is None:
+        q_lens = [ctx.host_q_start[i + 1] - ctx.host_q_start[i] for i in range(ctx.num_requests)]
+        row_tiles = 2 if ctx.max_q_len * group > 16 else 1
+        tile_req, tile_row0 = ops.attention_tiles(q_lens, group, row_tiles)
+        tiles = torch.tensor([tile_req, tile_row0], dtype=torch.int32).to(ctx.device)
+        split = ops.attention_split(ctx.max_kv_len, len(tile_req), nkv)
+        plan = AttentionPlan(tiles[0], tiles[1], row_tiles, ctx.max_kv_len, split)
+        ctx.extras[key] = plan
+    return plan
 
 
 @MIXERS.register("paged_attention")
@@ -91,10 +118,19 @@ class PagedAttention(Mixer):
             qkv, ctx.positions, ctx.token_req, cache.block_table, cos, sin,
             cache.keys, cache.values, nq, nkv, d, cache.page_size, write_cache=cache.writable,
         )
-        attn = ops.paged_attention_generic(
-            qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
-            nq, nkv, d, cache.page_size, window=self.window, scale=self.scale,
-        )
+        if ops.attention_mfma_supports(qkv.dtype, d, cache.page_size):
+            plan = attention_plan(ctx, nq // nkv, nkv)
+            attn = ops.paged_attention_mfma(
+                qkv, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
+                plan.tile_req, plan.tile_row0, plan.row_tiles, nq, nkv, d, cache.page_size,
+                plan.max_kv_len, plan.split, window=self.window, scale=self.scale,
+            )
+        else:
+            # the true 32-bit path, and shapes the matrix-core kernel does not take
+            attn = ops.paged_attention_generic(
+                qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
+                nq, nkv, d, cache.page_size, window=self.window, scale=self.scale,
+            )
         if rows is not None:
             attn = ops.gather_rows(attn, rows)
         return self.out(attn, residual=residual)
