@@ -18,8 +18,8 @@
 //
 // Splits.  The keys of a tile are cut at absolute multiples of `split`; each
 // (tile, kv head, split) is one wavefront.  A tile with one split writes the
-// output; otherwise partial (max, sum, weighted values) go to scratch and
-// tk_attention_merge adds them in split order.
+// output; otherwise partial (max, sum, weighted values) go to scratch and a
+// second kernel adds them in split order.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -68,6 +68,47 @@ __device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int
   t.s_first = t.lo / a.split;
   t.s_last = t.hi / a.split;
   return t;
+}
+
+// The loads of one step of 32 keys.  Keys: lane (r, q) reads 8 values of key
+// kb + 16 blk + r for every 32-wide step over the head size.  Values: lane (r, q)
+// reads, for d = 16 dt + r, the 4 keys kb + 16 blk + 4q .. + 3.  Addresses are
+// clamped into the tile's key range [lo, hi], so a load past the end reads valid memory.
+template <int DT>
+struct StepRegs {
+  bf16x8_t kv[2][(DT + 1) / 2];
+  bf16x4_t vv[DT][2];
+};
+
+template <int DT>
+__device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, const int* table,
+                                          int kvh, int kb, int lo, int hi, int r, int q) {
+  constexpr int D = DT * 16;
+  constexpr int KS = (DT + 1) / 2;
+  const int P = a.P;
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const int kk = min(max(kb + blk * 16 + r, lo), hi);
+    const int page = table[kk / P];
+    const bf16_t* kp = a.kcache + ((size_t)((size_t)page * a.nkv + kvh) * P + (kk % P)) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + q * 8;
+      if (d0 < D) {
+        s.kv[blk][ks] = *(const bf16x8_t*)(kp + d0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s.kv[blk][ks][e] = (__bf16)0.f;
+      }
+    }
+    int kc = kb + blk * 16 + q * 4;
+    if (kc > hi) kc = hi & ~3;
+    if (kc + 3 < lo) kc = lo & ~3;
+    const int vpage = table[kc / P];
+    const bf16_t* vp = a.vcache + ((size_t)((size_t)vpage * a.nkv + kvh) * D + r) * P + (kc % P);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) s.vv[dt][blk] = *(const bf16x4_t*)(vp + (size_t)dt * 16 * P);
+  }
 }
 
 template <int DT, int RT>
@@ -121,50 +162,36 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
     for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
+  StepRegs<DT> cur;
+  if (k_begin < k_end) load_step<DT>(cur, a, table, kvh, k_begin, t.lo, t.hi, r, q);
   for (int kb = k_begin; kb < k_end; kb += 32) {
-    // keys: lane (r, q) reads 8 values of key kb + 16 blk + r for every 32-wide step
-    bf16x8_t kv[2][KS];
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      const int kk = min(max(kb + blk * 16 + r, t.lo), t.hi);
-      const int page = table[kk / P];
-      const bf16_t* kp = a.kcache + ((size_t)((size_t)page * a.nkv + kvh) * P + (kk % P)) * D;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = ks * 32 + q * 8;
-        if (d0 < D) {
-          kv[blk][ks] = *(const bf16x8_t*)(kp + d0);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) kv[blk][ks][e] = (__bf16)0.f;
-        }
-      }
-    }
-    // values: lane (r, q) reads, for d = 16 dt + r, keys kb + 16 blk + 4q .. + 3
+    // the next step's loads are in flight while this step is computed
+    StepRegs<DT> nxt;
+    load_step<DT>(nxt, a, table, kvh, kb + 32 < k_end ? kb + 32 : kb, t.lo, t.hi, r, q);
+
+    // values of keys outside the tile's range may be anything (a freed page): make them
+    // zero by masking their 16 bits
     bf16x8_t vv[DT];
-    {
-      const bf16_t* vp[2];
-      bool ok[2][4];
+    uint32_t keep[2][2];
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
-        const int k4 = kb + blk * 16 + q * 4;
-        int kc = k4;
-        if (kc > t.hi) kc = t.hi & ~3;
-        if (kc + 3 < t.lo) kc = t.lo & ~3;
-        const int page = table[kc / P];
-        vp[blk] = a.vcache + ((size_t)((size_t)page * a.nkv + kvh) * D + r) * P + (kc % P);
+    for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) ok[blk][j] = (k4 + j >= t.lo) && (k4 + j <= t.hi) && kc == k4;
+      for (int h = 0; h < 2; ++h) {
+        const int key = kb + blk * 16 + q * 4 + 2 * h;
+        const uint32_t lo16 = (key >= t.lo && key <= t.hi) ? 0x0000ffffu : 0u;
+        const uint32_t hi16 = (key + 1 >= t.lo && key + 1 <= t.hi) ? 0xffff0000u : 0u;
+        keep[blk][h] = lo16 | hi16;
       }
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-          const bf16x4_t x = *(const bf16x4_t*)(vp[blk] + (size_t)dt * 16 * P);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) vv[dt][blk * 4 + j] = ok[blk][j] ? x[j] : (__bf16)0.f;
-        }
-      }
+    for (int dt = 0; dt < DT; ++dt) {
+      union { bf16x4_t v[2]; uint32_t u[4]; bf16x8_t w; } x;
+      x.v[0] = cur.vv[dt][0];
+      x.v[1] = cur.vv[dt][1];
+      x.u[0] &= keep[0][0];
+      x.u[1] &= keep[0][1];
+      x.u[2] &= keep[1][0];
+      x.u[3] &= keep[1][1];
+      vv[dt] = x.w;
     }
 
 #pragma unroll
@@ -172,8 +199,8 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
       f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv[0][ks], qv[rt][ks], st[0], 0, 0, 0);
-        st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv[1][ks], qv[rt][ks], st[1], 0, 0, 0);
+        st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[0][ks], qv[rt][ks], st[0], 0, 0, 0);
+        st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[1][ks], qv[rt][ks], st[1], 0, 0, 0);
       }
       float sc[8];
       float mx = -INFINITY;
@@ -208,9 +235,11 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
         acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[dt], pb, acc[rt][dt], 0, 0, 0);
       }
     }
+    cur = nxt;
   }
 
   // acc[rt][dt][j] of lane (r, q) is O^T[d = 16 dt + 4q + j][row r]
+  const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     float l = l_run[rt];
@@ -230,7 +259,7 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
         *(uint2*)(op + dt * 16 + q * 4) = pk.u;
       }
     } else {
-      const size_t item = ((size_t)tile * a.nkv + kvh) * a.max_splits + (s - t.s_first);
+      const size_t item = item0 + (s - t.s_first);
       float* po = a.part_o + (item * (16 * RT) + rt * 16 + r) * D;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *(f32x4_t*)(po + dt * 16 + q * 4) = acc[rt][dt];
@@ -243,32 +272,44 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
   }
 }
 
-// Adds the partial results of a tile's splits in split order.
-template <int RT>
-__global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D) {
+// Adds the partial results of split tiles, always in split order.  One wavefront
+// per (tile, kv head, row); lane i first takes the statistics of split i, then
+// every lane sums one (or more) of the row's d outputs over the splits.
+__global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D, int rows_per_tile) {
   const int tile = blockIdx.x, kvh = blockIdx.y;
-  const TileRange t = tile_range(a, tile, 16 * RT);
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.z * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const TileRange t = tile_range(a, tile, rows_per_tile);
   const int nsp = t.s_last - t.s_first + 1;
   if (nsp == 1) return;
-  const int rows = min(16 * RT, t.n_rows - t.row0);
+  if (row >= min(rows_per_tile, t.n_rows - t.row0)) return;
   const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
-  for (int i = threadIdx.x; i < rows * D; i += blockDim.x) {
-    const int row = i / D, d = i - row * D;
-    float m = -INFINITY;
-    for (int sp = 0; sp < nsp; ++sp)
-      m = fmaxf(m, a.part_ml[((item0 + sp) * (16 * RT) + row) * 2]);
-    float l = 0.f, o = 0.f;
+  const float* ml = a.part_ml + (item0 * rows_per_tile + row) * 2;  // split sp is sp * rows_per_tile * 2 further
+  const size_t ml_step = (size_t)rows_per_tile * 2;
+  float m = -INFINITY;
+  for (int sp = lane; sp < nsp; sp += 64) m = fmaxf(m, ml[sp * ml_step]);
+  m = wave_max(m);
+  float l = 0.f;
+  for (int sp = lane; sp < nsp; sp += 64) {
+    const float ms = ml[sp * ml_step];
+    l += (ms == -INFINITY ? 0.f : __expf(ms - m)) * ml[sp * ml_step + 1];
+  }
+  l = wave_sum(l);
+  const float inv = 1.0f / l;
+  const int flat = t.row0 + row;
+  const int tok = flat / a.group, g = flat - tok * a.group;
+  bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
+  const float* po = a.part_o + (item0 * rows_per_tile + row) * D;
+  const size_t po_step = (size_t)rows_per_tile * D;
+  for (int d = lane; d < D; d += 64) {
+    float o = 0.f;
+#pragma unroll 8
     for (int sp = 0; sp < nsp; ++sp) {
-      const size_t base = (item0 + sp) * (16 * RT) + row;
-      const float ms = a.part_ml[base * 2];
-      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
-      l += w * a.part_ml[base * 2 + 1];
-      o += w * a.part_o[base * D + d];
+      const float ms = ml[sp * ml_step];
+      const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
+      o += w * po[sp * po_step + d];
     }
-    const int flat = t.row0 + row;
-    const int tok = flat / a.group, g = flat - tok * a.group;
-    a.out[(size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D + d] =
-        __float2bfloat16(o / l);
+    op[d] = __float2bfloat16(o * inv);
   }
 }
 
@@ -297,8 +338,8 @@ static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, hipStream_
 // tiles; `grid_splits` is an upper bound on the splits of any tile and
 // `max_splits` the number the scratch has room for (grid_splits <= max_splits).
 // part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
-// tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when
-// max_splits is 1).  merge != 0 also launches the merge of split tiles.
+// tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when max_splits
+// is 1).  Launches that share scratch must not overlap.
 extern "C" int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                                        const void* kcache, const void* vcache,
                                        const int* block_table, int table_stride,
@@ -332,10 +373,8 @@ extern "C" int tk_paged_attention_mfma(const void* q, int q_stride, void* out, i
   TK_REQUIRE(ok, "attention_mfma: no kernel for head size %d", d);
   TK_CHECK_LAUNCH("paged_attention_mfma");
   if (max_splits > 1) {
-    if (row_tiles == 1)
-      hipLaunchKernelGGL((attention_merge_kernel<1>), dim3(n_tiles, nkv), dim3(256), 0, stream, a, d);
-    else
-      hipLaunchKernelGGL((attention_merge_kernel<2>), dim3(n_tiles, nkv), dim3(256), 0, stream, a, d);
+    const int rows = 16 * row_tiles;
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_tiles, nkv, rows / 4), dim3(256), 0, stream, a, d, rows);
     TK_CHECK_LAUNCH("attention_merge");
   }
   return 0;

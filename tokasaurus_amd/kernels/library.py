@@ -14,7 +14,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
 from tokasaurus_amd.kernels import build as _build
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class KernelError(RuntimeError):

@@ -313,10 +313,43 @@ def attention_tiles(q_lens: list[int], group: int, row_tiles: int) -> tuple[list
     return tile_req, tile_row0
 
 
-def attention_split(max_kv_len: int, n_tiles: int, nkv: int, target_waves: int = 4096) -> int:
-    """Keys per split (a multiple of 128) so that about ``target_waves`` wavefronts share the work."""
-    per = max_kv_len * max(n_tiles * nkv, 1) / target_waves
-    return max(128, -(-int(per) // 128) * 128)
+def attention_split(max_kv_len: int, n_tiles: int, nkv: int) -> int:
+    """Keys per split (a multiple of 128).  With few tiles the keys are split so
+    that several thousand wavefronts share the work (measured best on an MI355X:
+    256 keys up to batch 8 at 8192 keys, 512 at batch 64); with thousands of
+    tiles (prompts) nothing is split."""
+    base = max(n_tiles * nkv, 1)
+    whole = -(-max(max_kv_len, 1) // 128) * 128
+    if base >= 2048:
+        return whole
+    per = -(-(max_kv_len * base // 8192) // 128) * 128
+    return min(whole, max(256, per))
+
+
+class AttentionScratch:
+    """Memory for the partial results of split tiles.  The buffers grow on demand
+    and are shared by the launches of one stream, which run one after the other."""
+
+    _shared: dict = {}
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self.part_o = torch.empty((0,), dtype=torch.float32, device=device)
+        self.part_ml = torch.empty((0,), dtype=torch.float32, device=device)
+
+    @classmethod
+    def shared(cls, device: torch.device) -> "AttentionScratch":
+        key = (device.type, device.index)
+        if key not in cls._shared:
+            cls._shared[key] = cls(device)
+        return cls._shared[key]
+
+    def take(self, n_o: int, n_ml: int):
+        if self.part_o.numel() < n_o:
+            self.part_o = torch.empty((n_o,), dtype=torch.float32, device=self.device)
+        if self.part_ml.numel() < n_ml:
+            self.part_ml = torch.empty((n_ml,), dtype=torch.float32, device=self.device)
+        return self.part_o, self.part_ml
 
 
 def paged_attention_mfma(
@@ -338,7 +371,7 @@ def paged_attention_mfma(
     window: int = 0,
     scale: float | None = None,
     out: torch.Tensor | None = None,
-    scratch: tuple[torch.Tensor, torch.Tensor] | None = None,
+    scratch: "AttentionScratch | None" = None,
 ) -> torch.Tensor:
     """Attention of every token of the batch over its request's pages on the
     matrix cores (bfloat16).  ``q`` is 2-d and its first nq*d columns are the
@@ -376,16 +409,10 @@ def paged_attention_mfma(
     max_splits = max(1, -(-max_kv_len // split))
     part_o = part_ml = None
     if max_splits > 1:
-        rows = 16 * row_tiles
-        items = n_tiles * nkv * max_splits * rows
-        if scratch is not None:
-            part_o, part_ml = scratch
-            _need(part_o.dtype == torch.float32 and part_ml.dtype == torch.float32
-                  and part_o.numel() >= items * head_dim and part_ml.numel() >= items * 2,
-                  "attention_mfma: scratch too small")
-        else:
-            part_o = torch.empty((items * head_dim,), dtype=torch.float32, device=q.device)
-            part_ml = torch.empty((items * 2,), dtype=torch.float32, device=q.device)
+        items = n_tiles * nkv * max_splits * 16 * row_tiles
+        if scratch is None:
+            scratch = AttentionScratch.shared(q.device)
+        part_o, part_ml = scratch.take(items * head_dim, items * 2)
     call(
         "tk_paged_attention_mfma",
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
