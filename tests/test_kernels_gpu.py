@@ -79,3 +79,54 @@ def test_attention_splits_agree():
     outs = [run_attention("mfma", case, q_lens, kv_lens, nq, nkv, d, page, 0, split=s).float() for s in (4096, 512, 128, 32)]
     for o in outs[1:]:
         assert torch.allclose(o, outs[0], atol=1e-2, rtol=1e-2)
+
+
+# --------------------------------------------------------------------------
+# sampling
+# --------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("vocab", [1000, 2048, 2049, 128256])
+def test_sample_greedy_and_temperature(vocab):
+    import plain_llama
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(vocab)
+    rows = 12
+    logits = torch.randn((rows, vocab), generator=g) * 3.0
+    logits[3, 17] = logits[3].max() + 1.0
+    logits[3, 900] = logits[3, 17]  # a tie: the lowest index wins
+    temps = [0.0, 0.8, 1.0, 0.0, 0.3, 2.0, 0.8, 0.8, 0.8, 1e-3, 0.8, 0.8]
+    us = [0.0, 0.0, 0.5, 0.1, 0.999999, 0.25, 0.75, 0.01, 0.99, 0.5, 0.33, 0.66]
+    slots = torch.arange(rows, dtype=torch.int32).flip(0).contiguous().cuda()
+    last = torch.full((rows,), -1, dtype=torch.int32).cuda()
+    ids, lps = ops.sample(logits.cuda(), torch.tensor(temps).cuda(), torch.tensor(us).cuda(), slots, last)
+    ids, lps = ids.cpu().tolist(), lps.cpu()
+    assert last.cpu().flip(0).tolist() == ids
+    for r in range(rows):
+        want, want_lp = plain_llama.sample(logits[r], temps[r], us[r])
+        if temps[r] == 0:
+            assert ids[r] == want
+        else:
+            # the cumulative sums are rounded differently: the chosen token's interval
+            # of the 64-bit cumulative distribution must hold u up to that rounding
+            cdf = torch.cumsum(torch.softmax(logits[r].double() / temps[r], -1), -1)
+            lo = float(cdf[ids[r] - 1]) if ids[r] > 0 else 0.0
+            assert lo - 1e-5 <= us[r] < float(cdf[ids[r]]) + 1e-5, (r, ids[r], want)
+        ref_lp = torch.log_softmax(logits[r].double() / (temps[r] if temps[r] > 0 else 1.0), -1)[ids[r]]
+        assert abs(float(lps[r]) - float(ref_lp)) < 1e-3 + 1e-4 * abs(float(ref_lp))
+    assert ids[3] == 17
+
+
+def test_sample_frequencies_follow_the_probabilities():
+    from tokasaurus_amd.kernels import ops
+
+    vocab, n = 50, 4000
+    g = torch.Generator().manual_seed(1)
+    row = torch.randn((vocab,), generator=g) * 2.0
+    logits = row[None, :].expand(n, vocab).contiguous().cuda()
+    u = torch.rand((n,), generator=g).cuda()
+    ids, _ = ops.sample(logits, torch.full((n,), 0.7).cuda(), u)
+    freq = torch.bincount(ids.cpu().long(), minlength=vocab).double() / n
+    probs = torch.softmax(row.double() / 0.7, -1)
+    assert float((freq - probs).abs().max()) < 0.03

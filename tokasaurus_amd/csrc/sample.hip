@@ -1,39 +1,41 @@
-// Sampling from 32-bit logits, one workgroup per row:
+// Sampling from 32-bit logits:
 //   temperature == 0: the index of the largest raw logit (the lowest index on a tie);
 //   temperature  > 0: p = softmax(logits / T) and the smallest index whose
 //                     cumulative probability exceeds the row's uniform number u.
 // Also the chosen token's log-probability under p (T treated as 1 when 0), and
 // optionally the token written to the request's slot for the next step's embedding.
+//
+// Two kernels, so that a few rows of a large vocabulary still fill the chip:
+//   sample_partial: one workgroup per (row, chunk of SM_CHUNK logits): the chunk's
+//                   maximum, its first index, and sum exp((x - max) / T);
+//   sample_finish:  one workgroup per row: joins the chunks in chunk order, finds
+//                   the chunk in which the cumulative mass passes u, and scans it.
 #include "common.h"
 
-#define SM_THREADS 1024
+#define SM_THREADS 256
+#define SM_PER_THREAD 8
+#define SM_CHUNK (SM_THREADS * SM_PER_THREAD)
+#define SM_MAX_CHUNKS 4096
 
-__global__ __launch_bounds__(SM_THREADS) void sample_kernel(
+__global__ __launch_bounds__(SM_THREADS) void sample_partial_kernel(
     const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ temperature,
-    const float* __restrict__ uniform, const int* __restrict__ slots, int* __restrict__ last_token,
-    int* __restrict__ out_ids, float* __restrict__ out_logprobs) {
+    float* __restrict__ part_max, float* __restrict__ part_sum, int* __restrict__ part_arg,
+    int n_chunks) {
   __shared__ float red[16];
-  __shared__ float wave_tot[16];
   __shared__ int red_i[16];
-  __shared__ int chosen;
-  __shared__ float cum[SM_THREADS];
-  const int row = blockIdx.x;
-  const int tid = threadIdx.x;
-  const int lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
   const float* x = logits + (size_t)row * ld;
   const float T = temperature[row];
   const float inv_t = T > 0.f ? 1.0f / T : 1.0f;
-
-  // contiguous segment of this thread
-  const int per = (vocab + SM_THREADS - 1) / SM_THREADS;
-  const int begin = min(tid * per, vocab), end = min(begin + per, vocab);
-
-  // maximum and its first index
+  const int begin = chunk * SM_CHUNK + tid * SM_PER_THREAD;
+  float v[SM_PER_THREAD];
   float best = -INFINITY;
   int best_i = vocab;
-  for (int i = begin; i < end; ++i) {
-    const float v = x[i];
-    if (v > best) { best = v; best_i = i; }
+#pragma unroll
+  for (int i = 0; i < SM_PER_THREAD; ++i) {
+    v[i] = begin + i < vocab ? x[begin + i] : -INFINITY;
+    if (v[i] > best) { best = v[i]; best_i = begin + i; }
   }
   float m = best;
   int mi = best_i;
@@ -48,46 +50,119 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
   m = red[0]; mi = red_i[0];
   for (int w = 1; w < SM_THREADS / TK_WAVE; ++w)
     if (red[w] > m || (red[w] == m && red_i[w] < mi)) { m = red[w]; mi = red_i[w]; }
-  __syncthreads();
-  const float row_max = m;
-  const int argmax = mi;
-
-  // sum of exp((x - max) / T): per thread, then per wave, then the whole row
   float local = 0.f;
-  for (int i = begin; i < end; ++i) local += expf((x[i] - row_max) * inv_t);
-  // inclusive scan inside the wavefront (segments are ordered by thread id)
-  float scan = local;
 #pragma unroll
-  for (int o = 1; o < TK_WAVE; o <<= 1) {
-    const float up = __shfl_up(scan, o, TK_WAVE);
-    if (lane >= o) scan += up;
+  for (int i = 0; i < SM_PER_THREAD; ++i) local += (v[i] == -INFINITY) ? 0.f : expf((v[i] - m) * inv_t);
+  const float total = block_sum(local, red);
+  if (tid == 0) {
+    const size_t o = (size_t)row * n_chunks + chunk;
+    part_max[o] = m;
+    part_sum[o] = total;
+    part_arg[o] = mi;
   }
-  if (lane == TK_WAVE - 1) wave_tot[wave] = scan;
-  __syncthreads();
-  float before = 0.f, total = 0.f;
-  for (int w = 0; w < SM_THREADS / TK_WAVE; ++w) {
-    if (w < wave) before += wave_tot[w];
-    total += wave_tot[w];
+}
+
+__global__ __launch_bounds__(SM_THREADS) void sample_finish_kernel(
+    const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ temperature,
+    const float* __restrict__ uniform, const float* __restrict__ part_max,
+    const float* __restrict__ part_sum, const int* __restrict__ part_arg, int n_chunks,
+    const int* __restrict__ slots, int* __restrict__ last_token, int* __restrict__ out_ids,
+    float* __restrict__ out_logprobs) {
+  __shared__ float cum[SM_MAX_CHUNKS];  // mass of chunks 0..c relative to the row maximum
+  __shared__ float red[16];
+  __shared__ float wave_tot[16];
+  __shared__ float row_max_s, total_s;
+  __shared__ int argmax_s, pick_chunk, chosen;
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & (TK_WAVE - 1), wave = tid / TK_WAVE;
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row];
+  const float inv_t = T > 0.f ? 1.0f / T : 1.0f;
+  const float* pm = part_max + (size_t)row * n_chunks;
+  const float* ps = part_sum + (size_t)row * n_chunks;
+  const int* pa = part_arg + (size_t)row * n_chunks;
+
+  // the row's maximum and its first index
+  float m = -INFINITY;
+  int mi = vocab;
+  for (int c = tid; c < n_chunks; c += SM_THREADS) {
+    const float cm = pm[c];
+    const int ci = pa[c];
+    if (cm > m || (cm == m && ci < mi)) { m = cm; mi = ci; }
   }
-  // cum[i]: mass of the segments of threads 0..i.  Thread i owns the interval
-  // [cum[i-1], cum[i]); the intervals tile [0, cum[last]) without gaps.
-  cum[tid] = before + scan;
-  if (tid == 0) chosen = (T > 0.f) ? vocab - 1 : argmax;
+#pragma unroll
+  for (int o = TK_WAVE / 2; o > 0; o >>= 1) {
+    const float om = __shfl_xor(m, o, TK_WAVE);
+    const int oi = __shfl_xor(mi, o, TK_WAVE);
+    if (om > m || (om == m && oi < mi)) { m = om; mi = oi; }
+  }
+  __shared__ int red_i[16];
+  if (lane == 0) { red[wave] = m; red_i[wave] = mi; }
   __syncthreads();
+  if (tid == 0) {
+    float bm = red[0];
+    int bi = red_i[0];
+    for (int w = 1; w < SM_THREADS / TK_WAVE; ++w)
+      if (red[w] > bm || (red[w] == bm && red_i[w] < bi)) { bm = red[w]; bi = red_i[w]; }
+    row_max_s = bm;
+    argmax_s = bi;
+  }
+  __syncthreads();
+  const float row_max = row_max_s;
+  // every chunk's mass relative to the row maximum, then the running sum in chunk order
+  for (int c = tid; c < n_chunks; c += SM_THREADS) cum[c] = ps[c] * expf((pm[c] - row_max) * inv_t);
+  __syncthreads();
+  if (tid == 0) {
+    float run = 0.f;
+    for (int c = 0; c < n_chunks; ++c) { run += cum[c]; cum[c] = run; }
+    total_s = run;
+    pick_chunk = n_chunks - 1;
+    chosen = (T > 0.f) ? vocab - 1 : argmax_s;
+  }
+  __syncthreads();
+  const float total = total_s;
   if (T > 0.f) {
     const float target = uniform[row] * total;
-    const float lower = tid > 0 ? cum[tid - 1] : 0.f;
-    if (lower <= target && target < cum[tid] && begin < end) {
-      float c = lower;
-      int pick = end - 1;
-      for (int i = begin; i < end; ++i) {
-        c += expf((x[i] - row_max) * inv_t);
-        if (c > target) { pick = i; break; }
+    for (int c = tid; c < n_chunks; c += SM_THREADS) {
+      const float lower = c > 0 ? cum[c - 1] : 0.f;
+      if (lower <= target && target < cum[c]) atomicMin(&pick_chunk, c);
+    }
+    __syncthreads();
+    const int c = pick_chunk;
+    const float base = c > 0 ? cum[c - 1] : 0.f;
+    const int begin = c * SM_CHUNK + tid * SM_PER_THREAD;
+    float e[SM_PER_THREAD];
+    float local = 0.f;
+#pragma unroll
+    for (int i = 0; i < SM_PER_THREAD; ++i) {
+      e[i] = begin + i < vocab ? expf((x[begin + i] - row_max) * inv_t) : 0.f;
+      local += e[i];
+    }
+    float scan = local;  // inclusive scan over the threads, in thread order
+#pragma unroll
+    for (int o = 1; o < TK_WAVE; o <<= 1) {
+      const float up = __shfl_up(scan, o, TK_WAVE);
+      if (lane >= o) scan += up;
+    }
+    if (lane == TK_WAVE - 1) wave_tot[wave] = scan;
+    __syncthreads();
+    float before = base;
+    for (int w = 0; w < wave; ++w) before += wave_tot[w];
+    const float upper = before + scan, lower = upper - local;
+    // the last element of the chunk takes what rounding leaves over
+    const bool last_thread = begin < vocab && begin + SM_PER_THREAD >= min(vocab, (c + 1) * SM_CHUNK);
+    if (begin < vocab && lower <= target && (target < upper || last_thread)) {
+      float run = lower;
+      int pick = min(begin + SM_PER_THREAD, vocab) - 1;
+#pragma unroll
+      for (int i = 0; i < SM_PER_THREAD; ++i) {
+        run += e[i];
+        if (run > target && begin + i < vocab) { pick = min(pick, begin + i); }
       }
       atomicMin(&chosen, pick);
     }
+    __syncthreads();
   }
-  __syncthreads();
   if (tid == 0) {
     const int id = chosen;
     out_ids[row] = id;
@@ -96,14 +171,27 @@ __global__ __launch_bounds__(SM_THREADS) void sample_kernel(
   }
 }
 
+extern "C" int tk_sample_chunks(int vocab) { return (vocab + SM_CHUNK - 1) / SM_CHUNK; }
+
+// part_max, part_sum (float) and part_arg (int) hold rows * tk_sample_chunks(vocab) entries each.
 extern "C" int tk_sample(const float* logits, int ld, int rows, int vocab, const float* temperature,
                          const float* uniform, const int* slots, int* last_token, int* out_ids,
-                         float* out_logprobs, hipStream_t stream) {
+                         float* out_logprobs, float* part_max, float* part_sum, int* part_arg,
+                         hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "sample: bad sizes rows=%d vocab=%d ld=%d", rows,
              vocab, ld);
+  const int n_chunks = (vocab + SM_CHUNK - 1) / SM_CHUNK;
+  TK_REQUIRE(n_chunks <= SM_MAX_CHUNKS, "sample: a vocabulary of %d is larger than %d", vocab,
+             SM_MAX_CHUNKS * SM_CHUNK);
+  TK_REQUIRE(rows < 65536, "sample: %d rows are too many for one call", rows);
+  TK_REQUIRE(part_max && part_sum && part_arg, "sample: scratch missing");
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, vocab,
-                     temperature, uniform, slots, last_token, out_ids, out_logprobs);
-  TK_CHECK_LAUNCH("sample");
+  hipLaunchKernelGGL(sample_partial_kernel, dim3(n_chunks, rows), dim3(SM_THREADS), 0, stream, logits,
+                     ld, vocab, temperature, part_max, part_sum, part_arg, n_chunks);
+  TK_CHECK_LAUNCH("sample_partial");
+  hipLaunchKernelGGL(sample_finish_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, vocab,
+                     temperature, uniform, part_max, part_sum, part_arg, n_chunks, slots, last_token,
+                     out_ids, out_logprobs);
+  TK_CHECK_LAUNCH("sample_finish");
   return 0;
 }

@@ -10,7 +10,7 @@ import math
 
 import torch
 
-from tokasaurus_amd.kernels.library import KernelError, call
+from tokasaurus_amd.kernels.library import KernelError, call, load
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -451,6 +451,8 @@ def sample(
         _need(slots.numel() == rows, "sample: one slot a row")
     ids = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     logprobs = torch.empty((rows,), dtype=torch.float32, device=logits.device) if want_logprobs else None
+    chunks = load().tk_sample_chunks(vocab)
+    part = torch.empty((3, max(rows, 1) * chunks), dtype=torch.float32, device=logits.device)
     call(
         "tk_sample",
         logits.data_ptr(),
@@ -463,6 +465,9 @@ def sample(
         last_token.data_ptr() if last_token is not None else None,
         ids.data_ptr(),
         logprobs.data_ptr() if logprobs is not None else None,
+        part[0].data_ptr(),
+        part[1].data_ptr(),
+        part[2].data_ptr(),
         _stream(),
     )
     return ids, logprobs
