@@ -62,7 +62,7 @@ def parse() -> argparse.Namespace:
     return p.parse_args()
 
 
-def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int):
+def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int, context: int, use_graphs: bool):
     import torch
 
     from tokasaurus_amd.engine.runner import DTYPES, ModelRunner, require_gpu
@@ -76,7 +76,8 @@ def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int):
     model.load(tensors, DTYPES[dtype], device)
     del tensors
     torch.cuda.empty_cache()
-    return ModelRunner(model, PAGE_SIZE, num_tokens // PAGE_SIZE, max_slots)
+    return ModelRunner(model, PAGE_SIZE, num_tokens // PAGE_SIZE, max_slots, max_tokens_per_request=context,
+                       use_graphs=use_graphs, graph_max_size=max(128, max_slots))
 
 
 def make_engine(runner, args, max_seqs: int):
@@ -187,7 +188,8 @@ def main() -> int:
         cfgd["num_hidden_layers"] = args.layers
     points = [int(b) for b in args.points.split(",") if b]
     max_batch = max([args.batch] + points)
-    runner = build_runner(cfgd, args.dtype, num_tokens=max_batch * args.context, max_slots=max_batch)
+    runner = build_runner(cfgd, args.dtype, num_tokens=max_batch * args.context, max_slots=max_batch,
+                          context=args.context, use_graphs=not args.eager)
     elem = 2 if args.dtype == "bfloat16" else 4
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
 

@@ -16,6 +16,8 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import numpy as np
+
 from tokasaurus_amd.cache.pages import NoSpaceException, PagePool, SlotAllocator
 from tokasaurus_amd.parts.base import CacheNeed
 
@@ -70,7 +72,14 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, groups: list[CacheGroup], num_pages: int | list[int], page_size: int, max_slots: int):
+    def __init__(
+        self,
+        groups: list[CacheGroup],
+        num_pages: int | list[int],
+        page_size: int,
+        max_slots: int,
+        max_blocks_per_request: int | None = None,
+    ):
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         self.groups = groups
@@ -79,6 +88,17 @@ class CacheManager:
         self.pools = [PagePool(n) for n in counts]
         self.slots = SlotAllocator(max_slots)
         self.requests: dict[str, RequestCache] = {}
+        # Per group, the block tables once more as one array indexed by slot, kept
+        # up to date as pages come and go: a step whose shape is fixed (a recorded
+        # decode step) gathers its rows from it instead of walking lists.  Row
+        # `max_slots` belongs to no request: all its entries name the null page
+        # (the page after the pool's last), where padding rows of a step write.
+        self.max_blocks_per_request = max_blocks_per_request
+        self.slot_tables: list[np.ndarray] | None = None
+        if max_blocks_per_request is not None:
+            self.slot_tables = [
+                np.full((max_slots + 1, max_blocks_per_request), n, dtype=np.int32) for n in counts
+            ]
 
     # ---- arithmetic
     def blocks_for(self, num_tokens: int) -> int:
@@ -117,8 +137,16 @@ class CacheManager:
                     f"request {request_id!r} needs {need} more pages for {new_len} tokens, "
                     f"free: {self.num_free_pages()}"
                 )
-        for table, n, pool in zip(rc.tables, need, self.pools):
-            table.extend(pool.allocate(n))
+        if self.max_blocks_per_request is not None and self.blocks_for(new_len) > self.max_blocks_per_request:
+            raise ValueError(
+                f"request {request_id!r} would hold {new_len} tokens, more than the "
+                f"{self.max_blocks_per_request * self.page_size} a request may hold"
+            )
+        for g, (table, n, pool) in enumerate(zip(rc.tables, need, self.pools)):
+            new = pool.allocate(n)
+            if self.slot_tables is not None and new:
+                self.slot_tables[g][rc.slot, len(table) : len(table) + len(new)] = new
+            table.extend(new)
         rc.reserved_tokens = self.blocks_for(new_len) * self.page_size
 
     def advance(self, request_id: str, new_len: int) -> None:
@@ -143,6 +171,8 @@ class CacheManager:
                 if table[b] != RELEASED:
                     gone.append(table[b])
                     table[b] = RELEASED
+                    if self.slot_tables is not None:
+                        self.slot_tables[g][rc.slot, b] = self.pools[g].num_pages
             if gone:
                 self.pools[g].free(gone)
             rc.first_held[g] = max(rc.first_held[g], min(first_needed, len(table)))
@@ -152,6 +182,9 @@ class CacheManager:
         rc = self.requests.pop(request_id)
         for table, pool in zip(rc.tables, self.pools):
             pool.free([p for p in table if p != RELEASED])
+        if self.slot_tables is not None:
+            for g, pool in enumerate(self.pools):
+                self.slot_tables[g][rc.slot, :] = pool.num_pages
         self.slots.free(rc.slot)
 
     # ---- invariants (the reference's sanity_checks, allocator.py:158-194, without the tree)
@@ -168,3 +201,11 @@ class CacheManager:
         assert len(slots) == len(set(slots)), "a slot is held by two requests"
         for rc in self.requests.values():
             assert rc.num_tokens <= rc.reserved_tokens
+            if self.slot_tables is not None:
+                for g, table in enumerate(rc.tables):
+                    null = self.pools[g].num_pages
+                    row = self.slot_tables[g][rc.slot]
+                    want = [null if p == RELEASED else p for p in table]
+                    assert row[: len(table)].tolist() == want and (row[len(table) :] == null).all(), (
+                        f"group {g}: the slot table of request {rc.request_id!r} differs from its block table"
+                    )

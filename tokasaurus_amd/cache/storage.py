@@ -5,7 +5,9 @@ Per group: keys ``[entries, pages, nkv, P, d]`` and values
 the key rows of a page and the value columns of a page are contiguous for the
 attention kernels).  The reference keeps ``[pages, P, nkv, d]`` per layer for both
 (tokasaurus/model/kv_cache.py:27-54).  Per run entry with fixed-size state:
-``[slots, *shape]``.
+``[slots + 1, *shape]``.  The last page of every pool and the last slot belong to
+no request: rows that only pad a step to a recorded size write there (the
+reference's scratch page, tokasaurus/model/utils.py:363-369,552-554).
 """
 
 from __future__ import annotations
@@ -32,13 +34,15 @@ class CacheStorage:
         self.values: list[torch.Tensor] = []
         for grp, n in zip(groups, num_pages):
             nkv, d = grp.need.num_kv_heads, grp.need.head_dim
-            self.keys.append(torch.zeros((len(grp.entries), n, nkv, page_size, d), dtype=dtype, device=device))
-            self.values.append(torch.zeros((len(grp.entries), n, nkv, d, page_size), dtype=dtype, device=device))
+            # one page more than the pool hands out: the null page, where padding rows write
+            self.keys.append(torch.zeros((len(grp.entries), n + 1, nkv, page_size, d), dtype=dtype, device=device))
+            self.values.append(torch.zeros((len(grp.entries), n + 1, nkv, d, page_size), dtype=dtype, device=device))
         self.states: list[torch.Tensor | None] = [
-            torch.zeros((max_slots, *need.shape), dtype=need.dtype, device=device) if need is not None else None
+            torch.zeros((max_slots + 1, *need.shape), dtype=need.dtype, device=device) if need is not None else None
             for need in state_needs
         ]
-        self.last_token = torch.zeros((max_slots,), dtype=torch.int32, device=device)
+        # slot `max_slots` belongs to no request (padding rows of a recorded step use it)
+        self.last_token = torch.zeros((max_slots + 1,), dtype=torch.int32, device=device)
 
     def bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.keys + self.values)

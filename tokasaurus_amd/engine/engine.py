@@ -20,9 +20,9 @@ import torch
 
 from tokasaurus_amd.config.engine_config import EngineConfig
 from tokasaurus_amd.engine.batch import StepEntry
-from tokasaurus_amd.engine.runner import ModelRunner
+from tokasaurus_amd.engine.runner import ModelRunner, Sampling
 from tokasaurus_amd.engine.scheduler import Decision, Request, Scheduler
-from tokasaurus_amd.sampling import Sampler, SamplingParams, uniform_for
+from tokasaurus_amd.sampling import SamplingParams, uniform_for
 
 
 @dataclass
@@ -80,6 +80,10 @@ class Engine:
                 num_pages=config.kv_cache_num_blocks(),
                 max_slots=config.max_seqs_per_forward,
                 rope_scaling_override=config.rope_scaling_override(),
+                max_tokens_per_request=config.max_num_tokens_per_request,
+                use_graphs=config.use_hipgraphs,
+                graph_max_size=config.hipgraph_max_size,
+                graph_step=config.hipgraph_step,
             )
         else:
             config.finalize(runner.max_positions)
@@ -95,7 +99,6 @@ class Engine:
             max_prefill_chunk=config.max_prefill_chunk,
             sanity_checks=config.allocator_sanity_checks,
         )
-        self.sampler = Sampler(runner.model.device, want_logprobs=config.enable_chosen_logprobs)
         self.stats = Stats()
         self._next_id = 0
         self._request_seed: dict[str, int] = {}
@@ -140,20 +143,20 @@ class Engine:
             if self.scheduler.queued:
                 raise RuntimeError("requests are queued but none can be admitted: the cache is too small for them")
             return []
-        logits = self.runner.step(self._entries(decision))
         out_reqs = decision.requests_with_output()
+        # the rows of the step's output follow the entries: prompts that end, then decodes
+        temps = [r.params.temperature for r in out_reqs]
+        us = [
+            uniform_for(self.config.seed, self._request_seed[r.id], len(r.completion)) if r.params.temperature > 0 else 0.0
+            for r in out_reqs
+        ]
+        out = self.runner.run(self._entries(decision), Sampling(temps, us))
         tokens: list[int] = []
         logprobs: list[float] | None = None
         if out_reqs:
-            temps = [r.params.temperature for r in out_reqs]
-            us = [
-                uniform_for(self.config.seed, self._request_seed[r.id], len(r.completion)) if r.params.temperature > 0 else 0.0
-                for r in out_reqs
-            ]
-            slots = [self.runner.manager.requests[r.id].slot for r in out_reqs]
-            ids, lps = self.sampler.sample(logits, temps, us, slots, self.runner.storage.last_token)
-            tokens = ids.tolist()  # the step's one device-to-host synchronisation
-            logprobs = lps.tolist() if lps is not None else None
+            tokens = out.ids.tolist()  # the step's one device-to-host synchronisation
+            if self.config.enable_chosen_logprobs and out.logprobs is not None:
+                logprobs = out.logprobs.tolist()
         finished = self.scheduler.apply(decision, tokens, logprobs)
         self.stats.steps += 1
         self.stats.prefill_tokens += sum(n for _, n in decision.prefill)

@@ -10,16 +10,19 @@ top (the reference's forward never returns logits, tokasaurus/model/types.py:403
 
 from __future__ import annotations
 
+from dataclasses import dataclass
 from pathlib import Path
 
+import numpy as np
 import torch
 
 from tokasaurus_amd.cache.manager import CacheManager, plan_groups
 from tokasaurus_amd.cache.storage import CacheStorage
 from tokasaurus_amd.engine.batch import PlannedEntry, StepEntry, layout, to_device
+from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.models.causal_lm import CausalLM
 from tokasaurus_amd.models.registry import build_model, config_from_folder
-from tokasaurus_amd.parts.base import CacheView
+from tokasaurus_amd.parts.base import CacheView, StepContext
 from tokasaurus_amd.weights.loader import read_tensors
 
 DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -31,6 +34,153 @@ def require_gpu() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device())
 
 
+@dataclass
+class Sampling:
+    """One temperature and one uniform number for every wanted row of a step."""
+
+    temperatures: list[float]
+    uniforms: list[float]
+
+
+@dataclass
+class StepOutput:
+    logits: torch.Tensor  # [wanted, vocab] float32
+    ids: torch.Tensor | None = None  # [wanted] int32, when the step sampled
+    logprobs: torch.Tensor | None = None
+
+
+def graph_buckets(max_size: int, step: int) -> list[int]:
+    """Batch sizes decode steps are recorded at: 1, 2, 4, ... up to ``step``, then
+    multiples of ``step`` up to ``max_size`` (the reference pads to multiples of 16
+    up to 128, tokasaurus/common_types.py:117-121)."""
+    sizes = []
+    b = 1
+    while b < step and b <= max_size:
+        sizes.append(b)
+        b *= 2
+    sizes.extend(range(step, max_size + 1, step))
+    return sizes
+
+
+class RecordedDecodeStep:
+    """A decode step of fixed size (one token per request, padded to ``size`` rows)
+    recorded into a HIP graph: embedding, every block, the head and the sampler.
+
+    All of the step's integers and the sampler's numbers live in one device buffer
+    that is refilled by a single copy from pinned host memory before each replay.
+    Padding rows belong to no request: they read and write the null page and the
+    extra slot.  The step's attention is planned for the longest context a request
+    may have, so the same recording serves every length.
+    """
+
+    def __init__(self, runner: "ModelRunner", size: int):
+        self.runner = runner
+        self.size = size
+        model, storage, manager = runner.model, runner.storage, runner.manager
+        device = model.device
+        B = size
+        widths = [t.shape[1] for t in manager.slot_tables]
+        fields = [("token_ids", B), ("positions", B), ("token_req", B), ("q_start", B + 1), ("kv_len", B),
+                  ("slots", B), ("want_rows", B), ("temperature", B), ("uniform", B)]
+        fields += [(f"table{g}", B * w) for g, w in enumerate(widths)]
+        self.spans, at = {}, 0
+        for name, n in fields:
+            self.spans[name] = (at, n)
+            at += n
+        self.host = torch.zeros((at,), dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.host_f32 = self.host.view(torch.float32).numpy()
+        self.dev = torch.zeros((at,), dtype=torch.int32, device=device)
+        self.null_slot = manager.slots.num_slots
+        self._fill([], [], [], [], [], [])
+        self.dev.copy_(self.host)
+        self.copied = torch.cuda.Event()
+
+        def view(name: str) -> torch.Tensor:
+            a, n = self.spans[name]
+            return self.dev[a : a + n]
+
+        self.ctx = StepContext(
+            num_tokens=B, num_requests=B, dtype=model.dtype, device=device,
+            token_ids=view("token_ids"), positions=view("positions"), token_req=view("token_req"),
+            q_start=view("q_start"), kv_len=view("kv_len"), slots=view("slots"),
+            host_q_start=list(range(B + 1)), host_kv_len=[runner.max_tokens_per_request] * B, host_slots=[self.null_slot] * B,
+            last_token=storage.last_token, max_q_len=1, max_kv_len=runner.max_tokens_per_request,
+        )
+        self.ctx.extras["static"] = True  # parts keep what they plan: the step is replayed
+        self.ctx.extras["num_portions"] = 0
+        tables = [view(f"table{g}").view(B, w) for g, w in enumerate(widths)]
+        self.caches = runner.cache_views(tables)
+        self.want_rows = view("want_rows")
+        self.temperature = view("temperature").view(torch.float32)
+        self.uniform = view("uniform").view(torch.float32)
+
+        # once outside the graph (parts plan and allocate what they keep), then recorded
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            self._forward()
+        torch.cuda.current_stream().wait_stream(stream)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits, self.ids, self.logprobs = self._forward()
+        torch.cuda.synchronize()
+
+    def _forward(self):
+        logits = self.runner.model.forward(self.ctx, self.caches, self.runner.storage.states, self.want_rows)
+        ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.ctx.slots, self.runner.storage.last_token)
+        return logits, ids, logprobs
+
+    def _fill(self, token_ids, positions, slots, write_slots, temperatures, uniforms) -> None:
+        B, n = self.size, len(token_ids)
+        a = self.host_np
+        pad = B - n
+
+        def put(name, values, fill):
+            at, m = self.spans[name]
+            a[at : at + n] = values
+            a[at + n : at + m] = fill
+
+        put("token_ids", token_ids, 0)
+        put("positions", positions, 0)
+        put("kv_len", [p + 1 for p in positions], 1)
+        put("slots", write_slots, self.null_slot)
+        at, m = self.spans["token_req"]
+        a[at : at + m] = np.arange(m, dtype=np.int32)
+        at, m = self.spans["q_start"]
+        a[at : at + m] = np.arange(m, dtype=np.int32)
+        at, m = self.spans["want_rows"]
+        a[at : at + m] = np.arange(m, dtype=np.int32)
+        f = self.host_f32
+        at, m = self.spans["temperature"]
+        f[at : at + n] = temperatures
+        f[at + n : at + m] = 0.0
+        at, m = self.spans["uniform"]
+        f[at : at + n] = uniforms
+        f[at + n : at + m] = 0.0
+        rows = np.asarray(list(slots) + [self.null_slot] * pad, dtype=np.int64)
+        for g, table in enumerate(self.runner.manager.slot_tables):
+            at, m = self.spans[f"table{g}"]
+            a[at : at + m].reshape(B, table.shape[1])[:] = table[rows]
+
+    def run(self, planned: list[PlannedEntry], sampling: Sampling | None, write_slots: bool) -> StepOutput:
+        n = len(planned)
+        token_ids = [(-(e.slot + 1) if e.tokens is None else e.tokens[0]) for e in planned]
+        positions = [e.start for e in planned]
+        # a step that only wants logits must not disturb the requests' last tokens
+        slots = [e.slot for e in planned]
+        out_slots = slots if write_slots else [self.null_slot] * n
+        temps = sampling.temperatures if sampling is not None else [0.0] * n
+        us = sampling.uniforms if sampling is not None else [0.0] * n
+        self.copied.synchronize()  # the copy of the step before has read the host buffer
+        self._fill(token_ids, positions, slots, out_slots, temps, us)
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        self.graph.replay()
+        return StepOutput(self.logits[:n], self.ids[:n], self.logprobs[:n] if self.logprobs is not None else None)
+
+
 class ModelRunner:
     def __init__(
         self,
@@ -38,15 +188,31 @@ class ModelRunner:
         page_size: int,
         num_pages: int,
         max_slots: int,
+        max_tokens_per_request: int | None = None,
+        use_graphs: bool = True,
+        graph_max_size: int = 128,
+        graph_step: int = 16,
     ):
         assert model.device is not None, "load the model's weights first"
         self.model = model
         self.page_size = page_size
         self.max_positions = model.spec.max_positions
+        limit = min(self.max_positions, num_pages * page_size)
+        if max_tokens_per_request is not None:
+            limit = min(limit, max_tokens_per_request)
+        self.max_tokens_per_request = limit
         needs = model.cache_needs()
         cache_of = [e.cache_of for e in model.spec.run_order]
         self.groups, self.where = plan_groups(needs, cache_of)
-        self.manager = CacheManager(self.groups, num_pages, page_size, max_slots)
+        self.manager = CacheManager(
+            self.groups, num_pages, page_size, max_slots, max_blocks_per_request=-(-limit // page_size)
+        )
+        self.use_graphs = use_graphs
+        self.graph_sizes = [b for b in graph_buckets(graph_max_size, graph_step) if b <= max(max_slots, 1)] if use_graphs else []
+        if use_graphs and max_slots < graph_max_size and max_slots not in self.graph_sizes:
+            self.graph_sizes.append(max_slots)
+            self.graph_sizes.sort()
+        self.recorded: dict[int, RecordedDecodeStep] = {}
         self.storage = CacheStorage(
             self.groups,
             [num_pages] * len(self.groups),
@@ -67,6 +233,7 @@ class ModelRunner:
         num_pages: int,
         max_slots: int,
         rope_scaling_override: tuple[bool, dict | None] = (False, None),
+        **options,
     ) -> "ModelRunner":
         device = require_gpu()
         if dtype not in DTYPES:
@@ -78,7 +245,7 @@ class ModelRunner:
         allow = ("lm_head.weight",) if model.spec.head_name == model.spec.embedding_name else ()
         tensors = read_tensors(model_dir, specs, allow_unexpected=allow)
         model.load(tensors, DTYPES[dtype], device)
-        return cls(model, page_size, num_pages, max_slots)
+        return cls(model, page_size, num_pages, max_slots, **options)
 
     # ---- requests
     def admit(self, request_id: str) -> None:
@@ -97,20 +264,17 @@ class ModelRunner:
             rc = self.manager.requests[e.request_id]
             q_len = 1 if e.tokens is None else len(e.tokens)
             new_len = rc.num_tokens + q_len
-            if new_len > self.max_positions:
+            if new_len > self.max_tokens_per_request:
                 raise ValueError(
-                    f"request {e.request_id!r} would reach {new_len} tokens, the model's positions end at {self.max_positions}"
+                    f"request {e.request_id!r} would reach {new_len} tokens, a request may hold "
+                    f"{self.max_tokens_per_request} (the model's positions end at {self.max_positions})"
                 )
             self.manager.reserve(e.request_id, new_len)
             planned.append(PlannedEntry(e.request_id, e.tokens, list(e.want), rc.slot, rc.num_tokens, rc.tables))
         return planned
 
-    def step(self, entries: list[StepEntry]) -> torch.Tensor:
-        """Run one batch; logits [wanted, vocab] float32 in the order of the
-        entries and of their ``want`` lists."""
-        planned = self.plan(entries)
-        hb = layout(planned, self.model.spec.vocab_size, len(self.groups))
-        ctx, want_rows, tables = to_device(hb, self.model.dtype, self.model.device, self.storage.last_token)
+    def cache_views(self, tables: list[torch.Tensor]) -> list[CacheView | None]:
+        """For every run entry the pages it uses and its group's block table of this step."""
         caches: list[CacheView | None] = []
         for i, w in enumerate(self.where):
             if w is None:
@@ -126,7 +290,47 @@ class ModelRunner:
                     writable=self.model.spec.run_order[i].cache_of is None,
                 )
             )
-        logits = self.model.forward(ctx, caches, self.storage.states, want_rows)
+        return caches
+
+    def _recorded_for(self, planned: list[PlannedEntry]) -> RecordedDecodeStep | None:
+        """The recorded step that takes this batch: every request brings one
+        token and wants its logits, and a recorded size holds them."""
+        if not self.graph_sizes or not planned or len(planned) > self.graph_sizes[-1]:
+            return None
+        if any(e.q_len != 1 or e.want != [0] for e in planned):
+            return None
+        size = next(b for b in self.graph_sizes if b >= len(planned))
+        if size not in self.recorded:
+            self.recorded[size] = RecordedDecodeStep(self, size)
+        return self.recorded[size]
+
+    def run(self, entries: list[StepEntry], sampling: Sampling | None = None, write_slots: bool | None = None) -> StepOutput:
+        """Run one batch.  Logits [wanted, vocab] float32 come in the order of the
+        entries and of their ``want`` lists; with ``sampling`` every wanted row is
+        also sampled, and the token written to its request's slot."""
+        planned = self.plan(entries)
+        write_slots = (sampling is not None) if write_slots is None else write_slots
+        recorded = self._recorded_for(planned)
+        if recorded is not None:
+            out = recorded.run(planned, sampling, write_slots)
+        else:
+            hb = layout(planned, self.model.spec.vocab_size, len(self.groups))
+            ctx, want_rows, tables = to_device(hb, self.model.dtype, self.model.device, self.storage.last_token)
+            logits = self.model.forward(ctx, self.cache_views(tables), self.storage.states, want_rows)
+            out = StepOutput(logits)
+            if sampling is not None and logits.shape[0] > 0:
+                # rows are in the order of the entries' wants; one slot a row
+                slots = [e.slot for e in planned for _ in e.want]
+                dev = self.model.device
+                params = torch.tensor([sampling.temperatures, sampling.uniforms], dtype=torch.float32).to(dev)
+                slot_t = torch.tensor(slots, dtype=torch.int32).to(dev) if write_slots else None
+                out.ids, out.logprobs = ops.sample(
+                    logits, params[0], params[1], slot_t, self.storage.last_token if write_slots else None
+                )
         for e in planned:
             self.manager.advance(e.request_id, e.start + e.q_len)
-        return logits
+        return out
+
+    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Run one batch and return its logits only (nothing is sampled or written to slots)."""
+        return self.run(entries).logits
