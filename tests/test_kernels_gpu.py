@@ -130,3 +130,85 @@ def test_sample_frequencies_follow_the_probabilities():
     freq = torch.bincount(ids.cpu().long(), minlength=vocab).double() / n
     probs = torch.softmax(row.double() / 0.7, -1)
     assert float((freq - probs).abs().max()) < 0.03
+
+
+# --------------------------------------------------------------------------
+# matrix products
+# --------------------------------------------------------------------------
+
+
+def bf16_round(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).float()
+
+
+def gemm_reference(a, w, residual=None, swiglu=False, norm_weight=None, eps=0.0):
+    """32-bit reference with the roundings to bfloat16 where the engine stores bfloat16."""
+    a = a.double()
+    if norm_weight is not None:
+        # the kernel rounds a * weight once and scales by rstd at the end; the plain norm rounds
+        # the normalised value and its product with the weight: both are within a bfloat16 rounding of this
+        a = norm_weight.double() * (a * torch.rsqrt(a.pow(2).mean(-1, keepdim=True) + eps))
+    prod = a @ w.double().T
+    if swiglu:
+        inter = w.shape[0] // 2
+        g, u = bf16_round(prod[:, :inter].float()), bf16_round(prod[:, inter:].float())
+        return bf16_round(torch.nn.functional.silu(g)) * u
+    if residual is not None:
+        return bf16_round(prod.float()) + residual.float()
+    return prod.float()
+
+
+GEMM_SHAPES = [(2048, 256), (1000, 96), (777, 264), (48, 2048), (16, 32), (3072, 512)]  # (N, K)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 40, 64, 100, 128])
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+@pytest.mark.parametrize("mode", ["store", "residual", "f32", "swiglu", "norm_store", "norm_swiglu", "norm_f32_weight32"])
+def test_gemm_skinny(m, shape, mode):
+    from tokasaurus_amd.kernels import ops
+
+    n, k = shape
+    if "swiglu" in mode and n % 2:
+        n += 1
+    g = torch.Generator().manual_seed(m * 1000 + n + k)
+    a = (torch.randn((m, k), generator=g) * 1.5).to(torch.bfloat16)
+    w = (torch.randn((n, k), generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    kwargs, ref_kwargs = {}, {}
+    if mode == "residual":
+        res = torch.randn((m, n), generator=g).to(torch.bfloat16)
+        kwargs["residual"] = res.cuda()
+        ref_kwargs["residual"] = res
+    if "swiglu" in mode:
+        kwargs["swiglu"] = ref_kwargs["swiglu"] = True
+    if "f32" in mode:
+        kwargs["out_f32"] = True
+    if "norm" in mode:
+        nw = 1.0 + 0.1 * torch.randn((k,), generator=g)
+        nw = nw if mode.endswith("weight32") else nw.to(torch.bfloat16)
+        kwargs.update(norm_weight=nw.cuda(), norm_eps=1e-5)
+        ref_kwargs.update(norm_weight=nw, eps=1e-5)
+    ref = gemm_reference(a, w, **ref_kwargs)
+    for staged in ((0, 1) if m > 16 else (0,)):
+        got = ops.gemm_skinny_bf16(a.cuda(), w.cuda(), staged=staged, **kwargs).float().cpu()
+        assert got.shape == ref.shape
+        # 32-bit accumulation; a bfloat16 result is rounded to 8 bits, and a rounding of an
+        # intermediate (norm, gate, up) may fall the other way than in the reference
+        tol = dict(atol=2e-5, rtol=2e-5) if mode == "f32" else dict(atol=3e-2, rtol=2e-2)
+        if mode == "norm_f32_weight32":
+            tol = dict(atol=1e-2, rtol=1e-2)  # 32-bit output of a product of once-rounded inputs
+        err = (got - ref).abs()
+        bad = err > tol["atol"] + tol["rtol"] * ref.abs()
+        assert not bad.any(), f"staged={staged}: {int(bad.sum())} wrong, largest error {float(err.max()):.3e}"
+
+
+def test_gemm_rows_do_not_depend_on_the_batch():
+    """A token's outputs are the same bits whether it runs alone or among 100 others."""
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn((100, 512), generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn((1024, 512), generator=g) / 20).to(torch.bfloat16).cuda()
+    big = ops.gemm_skinny_bf16(a, w, out_f32=True)
+    for rows in (1, 7, 16, 33):
+        small = ops.gemm_skinny_bf16(a[:rows].contiguous(), w, out_f32=True)
+        assert torch.allclose(small, big[:rows], atol=1e-5, rtol=1e-5)

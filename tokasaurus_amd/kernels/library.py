@@ -14,7 +14,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
 from tokasaurus_amd.kernels import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class KernelError(RuntimeError):
@@ -39,7 +39,9 @@ _SIGNATURES: dict[str, list] = {
     "tk_paged_attention_mfma": [_P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P]
     + [c_int] * 7
     + [c_float, c_int, c_int, c_int, _P, _P, _P],
-    "tk_gemm_skinny_bf16": [_P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P],
+    "tk_gemm_skinny_bf16": [_P, c_int, _P, _P, c_int, _P, c_int, _P, c_int, c_float]
+    + [c_int] * 7
+    + [_P],
     "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
     "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
     "tk_sample_chunks": [c_int],

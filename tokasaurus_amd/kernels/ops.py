@@ -487,12 +487,16 @@ def gemm_skinny_bf16(
     residual: torch.Tensor | None = None,
     out_f32: bool = False,
     swiglu: bool = False,
+    norm_weight: torch.Tensor | None = None,
+    norm_eps: float = 0.0,
     waves_k: int = 0,
     tiles: int = 0,
+    staged: int = -1,
 ) -> torch.Tensor:
     """a [M <= 128, K] times w [N, K] transposed on the matrix cores, with the
     epilogue fused: + residual, 32-bit output, or (``swiglu``: w is [gate | up]
-    stacked, 2I rows) silu(gate) * up -> [M, I]."""
+    stacked, 2I rows) silu(gate) * up -> [M, I].  ``norm_weight``: ``a`` is
+    RMS-normed with this weight and ``norm_eps`` on the way in."""
     _gpu(a, w, residual)
     _need(a.dim() == 2 and a.stride(1) == 1 and a.dtype == torch.bfloat16, "gemm_skinny: A must be bfloat16 [M, K]")
     _need(w.dim() == 2 and w.is_contiguous() and w.dtype == torch.bfloat16, "gemm_skinny: W must be contiguous bfloat16 [N, K]")
@@ -510,13 +514,22 @@ def gemm_skinny_bf16(
         epi = EPI_RESIDUAL
     else:
         epi = EPI_F32 if out_f32 else EPI_STORE
+    if norm_weight is not None:
+        _gpu(norm_weight)
+        _need(norm_weight.shape == (k,) and norm_weight.is_contiguous()
+              and norm_weight.dtype in (torch.bfloat16, torch.float32),
+              "gemm_skinny: the norm weight must be contiguous [K], bfloat16 or float32")
+        _need(residual is None, "gemm_skinny: a norm in front cannot be combined with a residual behind")
     out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=a.device)
     call(
         "tk_gemm_skinny_bf16",
         a.data_ptr(), a.stride(0), w.data_ptr(), out.data_ptr(), n,
         residual.data_ptr() if residual is not None else None,
         residual.stride(0) if residual is not None else 0,
-        m, n, k, epi, waves_k, tiles, _stream(),
+        norm_weight.data_ptr() if norm_weight is not None else None,
+        1 if (norm_weight is not None and norm_weight.dtype == torch.float32) else 0,
+        float(norm_eps),
+        m, n, k, epi, waves_k, tiles, staged, _stream(),
     )
     return out
 
