@@ -188,8 +188,8 @@ def test_gemm_skinny(m, shape, mode):
         kwargs.update(norm_weight=nw.cuda(), norm_eps=1e-5)
         ref_kwargs.update(norm_weight=nw, eps=1e-5)
     ref = gemm_reference(a, w, **ref_kwargs)
-    for staged in ((0, 1) if m > 16 else (0,)):
-        got = ops.gemm_skinny_bf16(a.cuda(), w.cuda(), staged=staged, **kwargs).float().cpu()
+    for staged, tile_rows in ((0, 16), (0, 8), (1, 0)) if m > 16 else ((0, 16), (0, 8)):
+        got = ops.gemm_skinny_bf16(a.cuda(), w.cuda(), staged=staged, tile_rows=tile_rows, **kwargs).float().cpu()
         assert got.shape == ref.shape
         # 32-bit accumulation; a bfloat16 result is rounded to 8 bits, and a rounding of an
         # intermediate (norm, gate, up) may fall the other way than in the reference
@@ -198,7 +198,7 @@ def test_gemm_skinny(m, shape, mode):
             tol = dict(atol=1e-2, rtol=1e-2)  # 32-bit output of a product of once-rounded inputs
         err = (got - ref).abs()
         bad = err > tol["atol"] + tol["rtol"] * ref.abs()
-        assert not bad.any(), f"staged={staged}: {int(bad.sum())} wrong, largest error {float(err.max()):.3e}"
+        assert not bad.any(), f"staged={staged} tile_rows={tile_rows}: {int(bad.sum())} wrong, largest error {float(err.max()):.3e}"
 
 
 def test_gemm_rows_do_not_depend_on_the_batch():

@@ -18,7 +18,7 @@ void tk_set_error(const char* fmt, ...) {
 
 extern "C" const char* tk_last_error() { return g_error; }
 
-extern "C" int tk_abi_version() { return 8; }
+extern "C" int tk_abi_version() { return 9; }
 
 // --------------------------------------------------------------------------
 // embedding: out[t, :] = table[id_t, :]; id_t < 0 names slot -id_t-1 of `last_token`

@@ -45,6 +45,7 @@ struct GemmArgs {
   int norm_w_f32;
   float eps;
   int M, N, K;  // N: outputs (for SwiGLU the intermediate size; W then has 2N rows, gate first)
+  int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
 };
 
 __device__ __forceinline__ float silu_mul_bf16(float g, float u) {
@@ -135,15 +136,18 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
   f32x4_t* red = (f32x4_t*)smem;
   float* sq = (float*)(red + (WK > 1 ? (size_t)WK * NT * MB * 64 : 0));
 
-  // rows of W this lane streams (clamped: rows past the end are masked at the store)
+  // rows of W this lane streams (clamped: rows past the end are masked at the store);
+  // with tiles of 8 rows the upper lanes have no row and hold zeros
+  const int TH = a.TH;
+  const bool has_row = r < TH;
   const bf16_t* wp[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     int row;
     if (EPI == EPI_SWIGLU) {
-      row = min(g * 16 + r, a.N - 1) + t * a.N;  // t = 0 gate, t = 1 up
+      row = min(g * TH + r, a.N - 1) + t * a.N;  // t = 0 gate, t = 1 up
     } else {
-      row = min((g * NT + t) * 16 + r, a.N - 1);
+      row = min((g * NT + t) * TH + r, a.N - 1);
     }
     wp[t] = a.W + (size_t)row * a.K + q * 8;
   }
@@ -168,7 +172,13 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t) w[u][t] = *(const bf16x8_t*)(wp[t] + (size_t)(ks + u) * 32);
+        for (int t = 0; t < NT; ++t) {
+          if (has_row) {
+            w[u][t] = *(const bf16x8_t*)(wp[t] + (size_t)(ks + u) * 32);
+          } else {
+            w[u][t] = zero8();
+          }
+        }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) av[u][mb] = *(const bf16x8_t*)(ap[mb] + (size_t)(ks + u) * 32);
       }
@@ -196,7 +206,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       w[t] = *(const bf16x8_t*)(wp[t] + off);
-      if (!k_ok) w[t] = zero8();
+      if (!k_ok || !has_row) w[t] = zero8();
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -253,8 +263,9 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
           if (NORM && mm == mb) total = ss[mm];
         }
     }
+    if (qq * 4 >= TH) continue;
     const float scale = NORM ? 1.0f / sqrtf(total / (float)a.K + a.eps) : 1.0f;
-    const int n = (EPI == EPI_SWIGLU ? g : g * NT + t) * 16 + qq * 4;
+    const int n = (EPI == EPI_SWIGLU ? g : g * NT + t) * TH + qq * 4;
     store4<EPI>(a, s0, s1, scale, token, n);
   }
 }
@@ -511,11 +522,13 @@ static bool launch_mb(const GemmArgs& a, int epi, bool norm, int NT, int groups,
 // C [M, N].  norm_w (may be null): RMSNorm weight [K] applied to A first, bfloat16 or
 // float (norm_w_f32).  waves_k: wavefronts (skinny) or wavefront rows (staged) that split
 // K inside a workgroup (0 = choose); tiles: weight tiles of 16 rows per wavefront, 1 or 2
-// (0 = choose; SwiGLU always pairs gate and up); staged: -1 = choose by M, 0 = skinny, 1 = staged.
+// (0 = choose; SwiGLU always pairs gate and up); staged: -1 = choose, 0 = skinny, 1 = staged;
+// tile_rows: weight rows of a tile that the skinny kernel uses, 16 or 8 (0 = choose).
 extern "C" int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, int ldc,
                                    const void* residual, int ldr, const void* norm_w,
                                    int norm_w_f32, float eps, int M, int N, int K, int epi,
-                                   int waves_k, int tiles, int staged, hipStream_t stream) {
+                                   int waves_k, int tiles, int staged, int tile_rows,
+                                   hipStream_t stream) {
   TK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
   TK_REQUIRE(M <= 128, "gemm_skinny: at most 128 rows, got %d", M);
   TK_REQUIRE(epi >= EPI_STORE && epi <= EPI_F32, "gemm_skinny: unknown epilogue %d", epi);
@@ -529,16 +542,17 @@ extern "C" int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* 
   GemmArgs a;
   a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.C = C; a.ldc = ldc;
   a.residual = (const bf16_t*)residual; a.ldr = ldr; a.norm_w = norm_w; a.norm_w_f32 = norm_w_f32;
-  a.eps = eps; a.M = M; a.N = N; a.K = K;
+  a.eps = eps; a.M = M; a.N = N; a.K = K; a.TH = 16;
+  TK_REQUIRE(tile_rows == 0 || tile_rows == 8 || tile_rows == 16, "gemm_skinny: tile_rows %d is not 0, 8 or 16", tile_rows);
   const bool norm = norm_w != nullptr;
 
   const int n16 = (N + 15) / 16;
   const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
   const int K32 = (K + 31) / 32;
   const int n16_units = epi == EPI_SWIGLU ? n16 : n16;
-  // measured on an MI355X: passing A through LDS pays for a wide output (the head), where many
-  // wavefronts of a workgroup share it; a narrow one needs every tile in a workgroup of its own
-  const bool use_staged = MB >= 2 && (staged < 0 ? (K32 >= 2 * ST_SC && n16_units >= 2048) : staged != 0);
+  // measured on an MI355X: passing A through LDS pays for a wide output (the head) from 5 rows on,
+  // where many wavefronts of a workgroup share it; a narrow one needs every tile in a workgroup of its own
+  const bool use_staged = (staged < 0 ? M > 4 && K32 >= 2 * ST_SC && n16_units >= 2048 : staged != 0);
   TK_REQUIRE(!(norm && epi == EPI_RESIDUAL), "gemm_skinny: a norm in front cannot be combined with a residual behind");
   int NT = epi == EPI_SWIGLU ? 2 : (tiles > 0 ? tiles : 1);
   TK_REQUIRE(NT == 1 || NT == 2, "gemm_skinny: tiles=%d outside 1..2", NT);
@@ -547,20 +561,25 @@ extern "C" int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* 
   if (use_staged) {
     const int groups = (units + ST_WN - 1) / ST_WN;
     int WK = waves_k;
-    if (WK <= 0) WK = (1024 + groups * ST_WN - 1) / (groups * ST_WN);  // about a thousand wavefronts
+    if (WK <= 0) {
+      WK = (1024 + groups * ST_WN - 1) / (groups * ST_WN);  // about a thousand wavefronts
+      if (WK < 2) WK = 2;                                   // two rows a workgroup measured best
+    }
     const int lds_cap = (128 * 1024) / (2 * ST_SC * MB * 1024);        // two buffers within 128 KB
     if (WK > lds_cap) WK = lds_cap;
     if (WK > K32 / ST_SC) WK = K32 / ST_SC;                            // at least a round each
     if (WK > 16 / ST_WN) WK = 16 / ST_WN;
     if (WK < 1) WK = 1;
     switch (MB) {
-      case 1: ok = false; break;
+      case 1: ok = launch_mb<1, true>(a, epi, norm, NT, groups, WK, stream); break;
       case 2: ok = launch_mb<2, true>(a, epi, norm, NT, groups, WK, stream); break;
       case 4: ok = launch_mb<4, true>(a, epi, norm, NT, groups, WK, stream); break;
       default: ok = launch_mb<8, true>(a, epi, norm, NT, groups, WK, stream); break;
     }
   } else {
-    const int groups = units;
+    // fewer tiles than compute units: tiles of 8 rows make twice the workgroups
+    a.TH = tile_rows > 0 ? tile_rows : ((MB == 1 && units < 256) ? 8 : 16);
+    const int groups = a.TH == 16 ? units : (epi == EPI_SWIGLU ? (N + 7) / 8 : ((N + 7) / 8 + NT - 1) / NT);
     int WK = waves_k;
     if (WK <= 0) {
       // a wavefront issues the loads of U steps together: best when that is all it has to do,

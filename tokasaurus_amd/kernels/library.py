@@ -14,7 +14,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 
 from tokasaurus_amd.kernels import build as _build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 
 class KernelError(RuntimeError):
@@ -40,7 +40,7 @@ _SIGNATURES: dict[str, list] = {
     + [c_int] * 7
     + [c_float, c_int, c_int, c_int, _P, _P, _P],
     "tk_gemm_skinny_bf16": [_P, c_int, _P, _P, c_int, _P, c_int, _P, c_int, c_float]
-    + [c_int] * 7
+    + [c_int] * 8
     + [_P],
     "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
     "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],

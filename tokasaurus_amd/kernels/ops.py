@@ -492,6 +492,7 @@ def gemm_skinny_bf16(
     waves_k: int = 0,
     tiles: int = 0,
     staged: int = -1,
+    tile_rows: int = 0,
 ) -> torch.Tensor:
     """a [M <= 128, K] times w [N, K] transposed on the matrix cores, with the
     epilogue fused: + residual, 32-bit output, or (``swiglu``: w is [gate | up]
@@ -529,7 +530,7 @@ def gemm_skinny_bf16(
         norm_weight.data_ptr() if norm_weight is not None else None,
         1 if (norm_weight is not None and norm_weight.dtype == torch.float32) else 0,
         float(norm_eps),
-        m, n, k, epi, waves_k, tiles, staged, _stream(),
+        m, n, k, epi, waves_k, tiles, staged, tile_rows, _stream(),
     )
     return out
 
