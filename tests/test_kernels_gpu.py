@@ -212,3 +212,177 @@ def test_gemm_rows_do_not_depend_on_the_batch():
     for rows in (1, 7, 16, 33):
         small = ops.gemm_skinny_bf16(a[:rows].contiguous(), w, out_f32=True)
         assert torch.allclose(small, big[:rows], atol=1e-5, rtol=1e-5)
+
+
+# --------------------------------------------------------------------------
+# memory-bound kernels
+# --------------------------------------------------------------------------
+
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed_gather_and_slot_tokens(dtype):
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn((301, 72), generator=g).to(DT[dtype])
+    last = torch.tensor([7, 300, 12], dtype=torch.int32)
+    ids = torch.tensor([5, 0, 300, -1, -3, 17, -2], dtype=torch.int32)  # -k-1 names slot k
+    out = ops.embed_gather(ids.cuda(), table.cuda(), last.cuda()).cpu()
+    want = table[torch.tensor([5, 0, 300, 7, 12, 17, 300])]
+    assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [64, 96, 1000, 2048])
+def test_rmsnorm(dtype, hidden):
+    import plain_llama
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(hidden)
+    x = (torch.randn((7, hidden), generator=g) * 3).to(DT[dtype])
+    w = (1 + 0.1 * torch.randn((hidden,), generator=g)).to(DT[dtype])
+    for eps in (1e-5, 1e-6):
+        got = ops.rmsnorm(x.cuda(), w.cuda(), eps).cpu()
+        want = plain_llama.rms_norm(x, w, eps)  # the reference's order of casts, in the storage type
+        tol = dict(atol=1e-5, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=1e-2)
+        assert torch.allclose(got.float(), want.float(), **tol)
+    # a 32-bit weight with bfloat16 rows (a checkpoint that stores its norms in 32-bit)
+    if dtype == "bfloat16":
+        got = ops.rmsnorm(x.cuda(), w.float().cuda(), 1e-5).cpu()
+        assert torch.allclose(got.float(), plain_llama.rms_norm(x, w, 1e-5).float(), atol=2e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu_gather_add(dtype):
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(3)
+    gu = torch.randn((5, 2 * 193), generator=g).to(DT[dtype])
+    got = ops.swiglu(gu.cuda()).cpu().float()
+    gate, up = gu[:, :193].float(), gu[:, 193:].float()
+    want = torch.nn.functional.silu(gate) * up
+    tol = dict(atol=1e-6, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=2e-2)
+    assert torch.allclose(got, want, **tol)
+    assert float(ops.swiglu(torch.zeros((2, 8), dtype=DT[dtype]).cuda()).abs().max()) == 0.0
+
+    src = torch.randn((9, 200), generator=g).to(DT[dtype])
+    idx = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    assert torch.equal(ops.gather_rows(src.cuda(), idx.cuda()).cpu(), src[idx.long()])
+    wide = src.cuda()[:, :120]  # rows with a stride
+    assert torch.equal(ops.gather_rows(wide, idx.cuda()).cpu(), src[idx.long(), :120])
+
+    y = torch.randn((9, 200), generator=g).to(DT[dtype])
+    want = (src.float() + y.float()).to(DT[dtype])
+    assert torch.equal(ops.add(src.cuda(), y.cuda()).cpu(), want)
+
+
+def test_rope_table():
+    import plain_llama
+    from tokasaurus_amd.parts.position import inverse_frequencies
+    from tokasaurus_amd.kernels import ops
+
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 64}
+    for d, theta, sc in ((32, 500000.0, scaling), (16, 10000.0, None), (48, 10000.0, {"rope_type": "linear", "factor": 4.0})):
+        inv = inverse_frequencies(d, theta, sc)
+        want_inv = plain_llama.rope_inverse_frequencies(d, theta, sc)
+        assert torch.allclose(inv, want_inv, rtol=1e-6, atol=0)
+        cos, sin = ops.rope_table(inv.cuda(), 300)
+        wc, ws = plain_llama.rope_tables(torch.arange(300), want_inv)
+        # 32-bit angles up to 300 radians: the device's sine differs from the host's by a few ulp of the angle
+        assert torch.allclose(cos.cpu(), wc[:, : d // 2], atol=2e-5, rtol=0)
+        assert torch.allclose(sin.cpu(), ws[:, : d // 2], atol=2e-5, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 8, 64, 16), (6, 2, 48, 16)])
+def test_rope_append(dtype, shape):
+    """Rotation of q and k against the plain formula, and the place of every key and value in the pages."""
+    import plain_llama
+    from tokasaurus_amd.kernels import ops
+
+    nq, nkv, d, page = shape
+    g = torch.Generator().manual_seed(d)
+    q_lens, starts = [5, 1, 9], [3, 40, 0]  # a portion after 3 tokens, a decode at 40, a fresh prompt
+    n = sum(q_lens)
+    qkv = torch.randn((n, (nq + 2 * nkv) * d), generator=g).to(DT[dtype])
+    positions = torch.tensor([s + j for ql, s in zip(q_lens, starts) for j in range(ql)], dtype=torch.int32)
+    token_req = torch.tensor([r for r, ql in enumerate(q_lens) for _ in range(ql)], dtype=torch.int32)
+    blocks = [-(-(s + ql) // page) for ql, s in zip(q_lens, starts)]
+    pages = sum(blocks) + 2
+    perm = torch.randperm(pages, generator=g).tolist()
+    table = torch.full((3, max(blocks)), -1, dtype=torch.int32)
+    at = 0
+    for r, b in enumerate(blocks):
+        table[r, :b] = torch.tensor(perm[at : at + b], dtype=torch.int32)
+        at += b
+    inv = plain_llama.rope_inverse_frequencies(d, 10000.0, None)
+    cos_t, sin_t = plain_llama.rope_tables(torch.arange(64), inv)
+    kc = torch.full((pages, nkv, page, d), 7.0).to(DT[dtype]).cuda()
+    vc = torch.full((pages, nkv, d, page), 7.0).to(DT[dtype]).cuda()
+    dev_qkv = qkv.cuda()
+    ops.rope_append(dev_qkv, positions.cuda(), token_req.cuda(), table.cuda(), cos_t[:, : d // 2].contiguous().cuda(),
+                    sin_t[:, : d // 2].contiguous().cuda(), kc, vc, nq, nkv, d, page)
+    out = dev_qkv.cpu()
+    q = qkv[:, : nq * d].view(n, nq, d)
+    k = qkv[:, nq * d : (nq + nkv) * d].view(n, nkv, d)
+    v = qkv[:, (nq + nkv) * d :].view(n, nkv, d)
+    cos, sin = cos_t[positions.long()], sin_t[positions.long()]
+    want_q = plain_llama.apply_rope(q, cos, sin)
+    want_k = plain_llama.apply_rope(k, cos, sin)
+    tol = dict(atol=1e-6, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=1e-2)
+    assert torch.allclose(out[:, : nq * d].view(n, nq, d).float(), want_q.float(), **tol)
+    assert torch.equal(out[:, nq * d :], qkv[:, nq * d :]), "k and v columns of the input must stay as they were"
+    kc, vc = kc.cpu(), vc.cpu()
+    written = torch.zeros((pages, page), dtype=torch.bool)
+    for t in range(n):
+        p, o = int(table[token_req[t], positions[t] // page]), int(positions[t]) % page
+        assert torch.allclose(kc[p, :, o, :].float(), want_k[t].float(), **tol), t
+        assert torch.equal(vc[p, :, :, o], v[t]), t
+        written[p, o] = True
+    assert bool((kc[~written[:, None, :, None].expand_as(kc)] == 7.0).all()), "a key was written where no token lives"
+    assert bool((vc.permute(0, 1, 3, 2)[~written[:, None, :, None].expand(pages, nkv, page, d)] == 7.0).all())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mnk", [(1, 1000, 96), (37, 77, 130), (130, 64, 64), (5, 512, 2048)])
+def test_gemm_generic(dtype, mnk):
+    from tokasaurus_amd.kernels import ops
+
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn((m, k), generator=g).to(DT[dtype])
+    w = (torch.randn((n, k), generator=g) / math.sqrt(k)).to(DT[dtype])
+    res = torch.randn((m, n), generator=g).to(DT[dtype])
+    ref = a.double() @ w.double().T
+    tol = dict(atol=2e-5, rtol=2e-5)
+    assert torch.allclose(ops.gemm_generic(a.cuda(), w.cuda(), out_f32=True).cpu().double(), ref, **tol)
+    got = ops.gemm_generic(a.cuda(), w.cuda(), residual=res.cuda()).cpu()
+    want = (ref.float().to(DT[dtype]).float() + res.float()).to(DT[dtype])
+    tol = dict(atol=2e-5, rtol=2e-5) if dtype == "float32" else dict(atol=3e-2, rtol=2e-2)
+    assert torch.allclose(got.float(), want.float(), **tol)
+
+
+def test_kernels_refuse_what_they_cannot_do():
+    from tokasaurus_amd.kernels import ops
+    from tokasaurus_amd.kernels.library import KernelError
+
+    a = torch.zeros((2, 12), dtype=torch.bfloat16).cuda()
+    w = torch.zeros((16, 12), dtype=torch.bfloat16).cuda()
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops.gemm_skinny_bf16(a, w)
+    with pytest.raises(KernelError, match="no CPU path"):
+        ops.rmsnorm(torch.zeros((2, 8)), torch.ones((8,)), 1e-5)
+    with pytest.raises(KernelError, match="float32 or bfloat16"):
+        ops.rmsnorm(torch.zeros((2, 8), dtype=torch.float16).cuda(), torch.ones((8,), dtype=torch.float16).cuda(), 1e-5)
+    assert not ops.attention_mfma_supports(torch.bfloat16, 40, 16)
+    assert not ops.attention_mfma_supports(torch.bfloat16, 64, 6)
+    assert not ops.attention_mfma_supports(torch.float32, 64, 16)
+    # the generic attention takes any head size (here 40) and an odd page size
+    q_lens, kv_lens = [3, 1], [11, 30]
+    case = make_paged_case(q_lens, kv_lens, 4, 2, 40, 6, seed=1, dtype=torch.float32)
+    ref = attention_reference(case, q_lens, kv_lens, 4, 2, 40)
+    got = run_attention("generic_f32", case, q_lens, kv_lens, 4, 2, 40, 6, 0).cpu()
+    assert torch.allclose(got, ref, atol=2e-5, rtol=1e-4)
