@@ -140,17 +140,28 @@ def attention_block(
     cos: torch.Tensor,
     sin: torch.Tensor,
     window: int | None = None,
+    shared_kv: tuple[torch.Tensor, torch.Tensor] | None = None,
+    kv_out: list | None = None,
 ) -> torch.Tensor:
-    """llama.py:218-287: norm, q/k/v, rotation, attention, o_proj, residual."""
+    """llama.py:218-287: norm, q/k/v, rotation, attention, o_proj, residual.
+
+    ``shared_kv`` (not used by Llama): rotated keys and values of an earlier
+    block that this one reads instead of computing its own; ``kv_out`` receives
+    this block's (keys, values)."""
     nq = cfg["num_attention_heads"]
     nkv = cfg.get("num_key_value_heads", nq)
     T = x.shape[0]
     h = rms_norm(x, w[f"{prefix}.input_layernorm.weight"], cfg["rms_norm_eps"])
     q = linear(h, w[f"{prefix}.self_attn.q_proj.weight"]).view(T, nq, -1)
-    k = linear(h, w[f"{prefix}.self_attn.k_proj.weight"]).view(T, nkv, -1)
-    v = linear(h, w[f"{prefix}.self_attn.v_proj.weight"]).view(T, nkv, -1)
     q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
+    if shared_kv is None:
+        k = linear(h, w[f"{prefix}.self_attn.k_proj.weight"]).view(T, nkv, -1)
+        v = linear(h, w[f"{prefix}.self_attn.v_proj.weight"]).view(T, nkv, -1)
+        k = apply_rope(k, cos, sin)
+    else:
+        k, v = shared_kv
+    if kv_out is not None:
+        kv_out.append((k, v))
     a = causal_attention(q, k, v, window=window).reshape(T, -1)
     return x + linear(a, w[f"{prefix}.self_attn.o_proj.weight"])
 
@@ -199,12 +210,15 @@ def forward_logits(
     first_position: int = 0,
     layer_order: list[int] | None = None,
     windows: dict[int, int] | None = None,
+    kv_from: dict[int, int] | None = None,
 ) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence (llama.py:644-667, 572-582).
 
     ``first_position`` shifts every position (used by the invariance tests);
     ``layer_order`` runs the layers in another order or twice (default 0..L-1);
-    ``windows`` maps a layer index to a sliding window (default: none).
+    ``windows`` maps a layer index to a sliding window (default: none);
+    ``kv_from`` maps a place in the order to an earlier place whose keys and
+    values it reads instead of its own (default: none).
     """
     d = cfg["hidden_size"] // cfg["num_attention_heads"]  # llama.py:158-159
     ids = torch.tensor(token_ids, dtype=torch.int64)
@@ -215,10 +229,12 @@ def forward_logits(
     )
     cos, sin = rope_tables(positions, inv_freq)
     order = layer_order if layer_order is not None else range(cfg["num_hidden_layers"])
-    for i in order:
+    kvs: list = []
+    for place, i in enumerate(order):
         prefix = f"model.layers.{i}"
         window = (windows or {}).get(i)
-        x = attention_block(x, w, prefix, cfg, cos, sin, window=window)
+        shared = kvs[kv_from[place]] if kv_from and place in kv_from else None
+        x = attention_block(x, w, prefix, cfg, cos, sin, window=window, shared_kv=shared, kv_out=kvs)
         x = swiglu_block(x, w, prefix, cfg)
     return lm_head(x, w, cfg)
 

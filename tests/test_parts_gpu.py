@@ -1,0 +1,280 @@
+"""Each part alone against its plain formula, and models put together from parts
+in ways Llama does not use: a mixer with state of its own, a run order that names
+a layer twice and shares a cache, layers with a sliding window."""
+
+import json
+import math
+
+import pytest
+import torch
+from safetensors import safe_open
+from safetensors.torch import save_file
+
+import plain_llama
+import toy_parts
+from gpu_common import TOL
+from replay_helpers import compare, portions, run_steps, tail_one_by_one, whole
+from test_replay_gpu import mixed_trace
+from tiny_models import CONFIG_A, CONFIG_B, random_tokens
+from tokasaurus_amd.engine.batch import PlannedEntry, layout, to_device
+from tokasaurus_amd.engine.runner import ModelRunner
+from tokasaurus_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, PartSpec
+from tokasaurus_amd.parts.embedding import LMHead, TokenEmbedding
+from tokasaurus_amd.parts.linear import Placer
+from tokasaurus_amd.weights import write_random_model
+
+pytestmark = pytest.mark.gpu
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# bfloat16: queries and keys are rounded to 8 bits after the rotation, which moves a score of
+# spread 3 by a few hundredths and a peaked softmax by a few percent (the same bound as the
+# replay tests use for logits)
+PART_TOL = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=6e-2, rtol=5e-2)}
+
+
+def rand(shape, g, dtype, scale=1.0):
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def context(q_lens, starts, tables, dtype, vocab=100):
+    """A step's context for requests that bring q_lens tokens after holding `starts`."""
+    planned = [PlannedEntry(f"r{i}", [1] * ql, [], slot=i, start=st, tables=[tab])
+               for i, (ql, st, tab) in enumerate(zip(q_lens, starts, tables))]
+    hb = layout(planned, vocab, 1)
+    ctx, _, dev_tables = to_device(hb, dtype, torch.device("cuda"), None)
+    return ctx, dev_tables[0]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_norm_feed_forward_embedding_and_head_alone(dtype):
+    g = torch.Generator().manual_seed(0)
+    H, I, V = 96, 200, 333
+    dt = DT[dtype]
+    placer = Placer(dt, torch.device("cuda"))
+    tensors = {
+        "n.weight": (1 + 0.1 * torch.randn((H,), generator=g)).to(dt),
+        "g.weight": rand((I, H), g, dt, 0.1), "u.weight": rand((I, H), g, dt, 0.1), "d.weight": rand((H, I), g, dt, 0.1),
+        "e.weight": rand((V, H), g, dt), "h.weight": rand((V, H), g, dt, 0.1),
+    }
+    f32 = {k: v.float() for k, v in tensors.items()}
+    x = rand((11, H), g, dt)
+    xf = x.float()
+
+    norm = NORMS.build(PartSpec("rmsnorm", {"size": H, "eps": 1e-6, "name": "n.weight"}))
+    assert [s.name for s in norm.tensor_specs()] == ["n.weight"]
+    norm.load(tensors, placer)
+    want = plain_llama.rms_norm(xf, f32["n.weight"], 1e-6)
+    assert torch.allclose(norm.forward(x.cuda()).cpu().float(), want, **PART_TOL[dtype])
+
+    ff = FEED_FORWARDS.build(PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I,
+                                                 "names": {"gate": "g.weight", "up": "u.weight", "down": "d.weight"}}))
+    ff.load(tensors, placer)
+    res = rand((11, H), g, dt)
+    gate, up = xf @ f32["g.weight"].T, xf @ f32["u.weight"].T
+    want = res.float() + (torch.nn.functional.silu(gate) * up) @ f32["d.weight"].T
+    assert torch.allclose(ff.forward(x.cuda(), res.cuda()).cpu().float(), want, **PART_TOL[dtype])
+
+    emb = TokenEmbedding(V, H, "e.weight")
+    emb.load(tensors, placer)
+    ctx, _ = context([3, 1], [0, 5], [[0], [1]], dt, vocab=V)
+    ctx.token_ids.copy_(torch.tensor([7, 0, 332, 100], dtype=torch.int32))
+    assert torch.equal(emb.forward(ctx).cpu(), tensors["e.weight"][[7, 0, 332, 100]])
+
+    head = LMHead(V, H, "h.weight", PartSpec("rmsnorm", {"size": H, "eps": 1e-6, "name": "n.weight"}))
+    head.load(tensors, placer)
+    got = head.forward(x.cuda())
+    assert got.dtype == torch.float32
+    want = plain_llama.rms_norm(xf, f32["n.weight"], 1e-6) @ f32["h.weight"].T
+    assert torch.allclose(got.cpu(), want, **PART_TOL[dtype])
+    # a tied head reads the embedding's buffer: placed once
+    tied = LMHead(V, H, "e.weight", PartSpec("rmsnorm", {"size": H, "eps": 1e-6, "name": "n.weight"}))
+    tied.load(tensors, placer)
+    assert tied.proj.weight.data_ptr() == emb.table.data_ptr()
+
+
+def test_rotary_encoding_alone():
+    scaling = CONFIG_B["rope_scaling"]
+    rot = POSITION_ENCODINGS.build(PartSpec("rotary", {"head_dim": 32, "theta": 500000.0, "max_positions": 200, "scaling": scaling}))
+    rot.prepare(torch.device("cuda"))
+    inv = plain_llama.rope_inverse_frequencies(32, 500000.0, scaling)
+    cos, sin = plain_llama.rope_tables(torch.arange(200), inv)
+    assert rot.cos.dtype == torch.float32 and tuple(rot.cos.shape) == (200, 16)
+    assert torch.allclose(rot.cos.cpu(), cos[:, :16], atol=2e-5) and torch.allclose(rot.sin.cpu(), sin[:, :16], atol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(64, 4, 2, 16, 4, 0), (96, 3, 1, 32, 8, 0), (256, 4, 1, 64, 16, 0), (96, 3, 1, 32, 8, 10)])
+def test_attention_mixer_and_block_alone(dtype, shape):
+    """One request in two steps (a portion, then the rest beside a second request):
+    the mixer and the whole block against the plain formulas on the whole sequences."""
+    H, nq, nkv, d, page, window = shape
+    I = 160
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(H + window)
+    names = {"q": "q.weight", "k": "k.weight", "v": "v.weight", "o": "o.weight"}
+    sharp = math.sqrt(3.0 / H)  # scores with a spread of about 3: a wrong key shows
+    tensors = {
+        "q.weight": rand((nq * d, H), g, dt, sharp), "k.weight": rand((nkv * d, H), g, dt, sharp),
+        "v.weight": rand((nkv * d, H), g, dt, 0.1), "o.weight": rand((H, nq * d), g, dt, 0.1),
+        "n1.weight": (1 + 0.1 * torch.randn((H,), generator=g)).to(dt), "n2.weight": (1 + 0.1 * torch.randn((H,), generator=g)).to(dt),
+        "g.weight": rand((I, H), g, dt, 0.1), "u.weight": rand((I, H), g, dt, 0.1), "d.weight": rand((H, I), g, dt, 0.1),
+    }
+    position = PartSpec("rotary", {"head_dim": d, "theta": 10000.0, "max_positions": 128, "scaling": None})
+    mixer_spec = PartSpec("paged_attention", {"hidden_size": H, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d,
+                                              "names": names, "position": position, "window": window})
+    block_spec = PartSpec("pre_norm", {
+        "mixer_norm": PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "name": "n1.weight"}), "mixer": mixer_spec,
+        "ff_norm": PartSpec("rmsnorm", {"size": H, "eps": 1e-5, "name": "n2.weight"}),
+        "feed_forward": PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I, "names": {"gate": "g.weight", "up": "u.weight", "down": "d.weight"}}),
+    })
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "rms_norm_eps": 1e-5}
+    w = {f"L.self_attn.{k}_proj.weight": tensors[f"{k}.weight"].float() for k in "qkvo"}
+    w.update({"L.input_layernorm.weight": tensors["n1.weight"].float(), "L.post_attention_layernorm.weight": tensors["n2.weight"].float(),
+              "L.mlp.gate_proj.weight": tensors["g.weight"].float(), "L.mlp.up_proj.weight": tensors["u.weight"].float(),
+              "L.mlp.down_proj.weight": tensors["d.weight"].float()})
+    inv = plain_llama.rope_inverse_frequencies(d, 10000.0, None)
+    lens = {"a": 41, "b": 9}
+    xs = {r: rand((n, H), g, dt) for r, n in lens.items()}
+
+    for part in ("mixer", "block"):
+        placer = Placer(dt, torch.device("cuda"))
+        built = (MIXERS if part == "mixer" else BLOCKS).build(mixer_spec if part == "mixer" else block_spec)
+        built.load(tensors, placer)
+        need = (built if part == "mixer" else built.mixer).cache_need()
+        assert (need.num_kv_heads, need.head_dim, need.window) == (nkv, d, window)
+        pages = 32
+        keys = torch.full((pages, nkv, page, d), float("nan"), dtype=dt, device="cuda")
+        values = torch.full((pages, nkv, d, page), float("nan"), dtype=dt, device="cuda")
+        perm = torch.randperm(pages, generator=g).tolist()
+        tab_a, tab_b = perm[: -(-lens["a"] // page)], perm[16 : 16 + -(-lens["b"] // page)]
+        got = {}
+        # step 1: 29 tokens of a; step 2: the other 12 of a beside all of b
+        for q_lens, starts, tabs, reqs in (([29], [0], [tab_a], ["a"]), ([12, 9], [29, 0], [tab_a, tab_b], ["a", "b"])):
+            ctx, table = context(q_lens, starts, tabs, dt)
+            cache = CacheView(keys, values, table, page)
+            x = torch.cat([xs[r][s : s + n] for r, s, n in zip(reqs, starts, q_lens)]).cuda()
+            if part == "mixer":
+                out = built.forward(x, x, ctx, cache, None, None)  # h = residual = x
+            else:
+                out = built.forward(x, ctx, cache, None, None)
+            at = 0
+            for r, s, n in zip(reqs, starts, q_lens):
+                got.setdefault(r, []).append(out[at : at + n].cpu().float())
+                at += n
+        for r, n in lens.items():
+            x = xs[r].float()
+            cos, sin = plain_llama.rope_tables(torch.arange(n), inv)
+            if part == "mixer":
+                q = plain_llama.apply_rope((x @ w["L.self_attn.q_proj.weight"].T).view(n, nq, d), cos, sin)
+                k = plain_llama.apply_rope((x @ w["L.self_attn.k_proj.weight"].T).view(n, nkv, d), cos, sin)
+                v = (x @ w["L.self_attn.v_proj.weight"].T).view(n, nkv, d)
+                a = plain_llama.causal_attention(q, k, v, window=window or None).reshape(n, -1)
+                want = x + a @ w["L.self_attn.o_proj.weight"].T
+            else:
+                want = plain_llama.attention_block(x, w, "L", cfg, cos, sin, window=window or None)
+                want = plain_llama.swiglu_block(want, w, "L", cfg)
+            err = (torch.cat(got[r]) - want).abs()
+            # an output is a sum of many rounded terms: its error scales with the typical size
+            # of the outputs, not with its own (terms cancel)
+            scale = want.abs() + (want.pow(2).mean().sqrt() if dtype == "bfloat16" else 0.0)
+            bound = PART_TOL[dtype]["atol"] + PART_TOL[dtype]["rtol"] * scale
+            assert bool((err <= bound).all()), (part, r, f"{int((err > bound).sum())} of {err.numel()} wrong, largest error {float(err.max()):.3e}, mean {float(err.mean()):.3e}")
+
+
+# --------------------------------------------------------------------------
+# models put together differently
+# --------------------------------------------------------------------------
+
+
+def sharpen(folder, scale_by_suffix):
+    path = folder / "model.safetensors"
+    tensors = {}
+    with safe_open(str(path), framework="pt") as f:
+        for name in f.keys():
+            t = f.get_tensor(name)
+            for suffix, scale in scale_by_suffix.items():
+                if name.endswith(suffix):
+                    t = (t.float() * scale).to(t.dtype)
+            tensors[name] = t
+    save_file(tensors, str(path))
+
+
+def all_cuttings(runner, reqs, ref, tol):
+    for k, (rid, toks) in enumerate(reqs.items()):
+        compare(run_steps(runner, whole(rid, toks)), ref, **tol)
+        if len(toks) > 32:
+            compare(run_steps(runner, tail_one_by_one(rid, toks, 32)), ref, **tol)
+        compare(run_steps(runner, portions(rid, toks, [[16, 7, 2, 5, 3], [2, 2, 31, 1, 4, 9]][k % 2])), ref, **tol)
+    got = run_steps(runner, mixed_trace(reqs, seed=5))
+    assert len(got) == sum(len(t) for t in reqs.values())
+    compare(got, ref, **tol)
+    runner.manager.check()
+    assert all(pool.num_free == pool.num_pages for pool in runner.manager.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_state_of_its_own(tmp_path, dtype):
+    """A toy recurrent mixer, defined in the tests, is registered, built from a
+    config.json, given random weights and stepped in every cutting."""
+    toy_parts.register()
+    config = dict(CONFIG_A, model_type="toy_recurrent", num_hidden_layers=3, toy_state_size=24, toy_recurrent_layers=[1])
+    folder = write_random_model(tmp_path / "toy", config, seed=4)
+    sharpen(folder, {"mixer.in.weight": 5.0, "mixer.out.weight": 5.0, "q_proj.weight": math.sqrt(3.0 / 64) / 0.02,
+                     "k_proj.weight": math.sqrt(3.0 / 64) / 0.02})
+    cfg, w = plain_llama.load_folder(folder)
+    reqs = {f"t{n}": random_tokens(n, cfg["vocab_size"], n) for n in (45, 70, 9, 38, 3)}
+    ref = {rid: toy_parts.plain_toy_recurrent_logits(cfg, w, toks) for rid, toks in reqs.items()}
+    # the state matters: without it the logits are far from these
+    no_state = dict(w)
+    no_state["model.layers.1.mixer.out.weight"] = torch.zeros_like(w["model.layers.1.mixer.out.weight"])
+    assert (toy_parts.plain_toy_recurrent_logits(cfg, no_state, reqs["t45"]) - ref["t45"]).abs().max() > 0.05
+    runner = ModelRunner.from_folder(folder, dtype, page_size=4, num_pages=64, max_slots=4)
+    assert [n is not None for n in runner.model.state_needs()] == [False, True, False]
+    assert [n is not None for n in runner.model.cache_needs()] == [True, False, True]
+    all_cuttings(runner, reqs, ref, TOL[dtype])
+    assert runner.recorded, "decode steps of the toy model were not recorded"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_run_order_as_data_and_a_shared_cache(tmp_path, dtype):
+    """Layer 0 runs twice (each use with a cache of its own) and the last entry
+    reads the cache of the second instead of keeping one."""
+    toy_parts.register()
+    order = [[0, None], [1, None], [0, None], [2, 1]]
+    config = dict(CONFIG_B, model_type="toy_arranged", toy_run_order=order)
+    folder = write_random_model(tmp_path / "arranged", config, seed=6)
+    sharpen(folder, {"q_proj.weight": math.sqrt(3.0 / 96) / 0.02, "k_proj.weight": math.sqrt(3.0 / 96) / 0.02})
+    cfg, w = plain_llama.load_folder(folder)
+    reqs = {f"o{n}": random_tokens(n, cfg["vocab_size"], n) for n in (50, 9, 77, 33)}
+    ref = {rid: toy_parts.plain_arranged_logits(cfg, w, toks) for rid, toks in reqs.items()}
+    assert (plain_llama.forward_logits(cfg, w, reqs["o50"]) - ref["o50"]).abs().max() > 0.05
+    runner = ModelRunner.from_folder(folder, dtype, page_size=8, num_pages=40, max_slots=4)
+    assert len(runner.groups) == 1 and runner.groups[0].entries == (0, 1, 2)  # three caches, the fourth entry shares
+    all_cuttings(runner, reqs, ref, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sliding_window_layers_have_pages_of_their_own(tmp_path, dtype):
+    """Layer 1 reads only the last 20 keys: its pages form a group of their own and
+    go back to the pool as the window passes them, while the request still runs."""
+    toy_parts.register()
+    config = dict(CONFIG_B, model_type="toy_arranged", toy_run_order=[[0, None], [1, None], [2, None]], toy_windows={"1": 20})
+    folder = write_random_model(tmp_path / "windowed", config, seed=8)
+    sharpen(folder, {"q_proj.weight": math.sqrt(3.0 / 96) / 0.02, "k_proj.weight": math.sqrt(3.0 / 96) / 0.02})
+    cfg, w = plain_llama.load_folder(folder)
+    reqs = {f"w{n}": random_tokens(n, cfg["vocab_size"], n) for n in (120, 9, 64, 41)}
+    ref = {rid: toy_parts.plain_arranged_logits(cfg, w, toks) for rid, toks in reqs.items()}
+    # the window's edge shows: the same weights without a window give other logits
+    assert (plain_llama.forward_logits(cfg, w, reqs["w120"]) - ref["w120"])[40:].abs().max() > 0.05
+    runner = ModelRunner.from_folder(folder, dtype, page_size=8, num_pages=40, max_slots=4)
+    assert sorted(grp.need.window for grp in runner.groups) == [0, 20]
+    gw = next(i for i, grp in enumerate(runner.groups) if grp.need.window == 20)
+    # while a long request decodes, the windowed group holds few pages and the full group all of them
+    toks = reqs["w120"]
+    steps = tail_one_by_one("w120", toks, 60)
+    steps[-1].pop("end")
+    got = run_steps(runner, steps)
+    compare(got, ref, **TOL[dtype])
+    held = [runner.manager.pools[i].num_pages - runner.manager.pools[i].num_free for i in range(2)]
+    assert held[1 - gw] == 15 and held[gw] <= 4, held
+    runner.release("w120")
+    all_cuttings(runner, reqs, ref, TOL[dtype])

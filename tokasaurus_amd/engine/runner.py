@@ -81,7 +81,7 @@ class RecordedDecodeStep:
         B = size
         widths = [t.shape[1] for t in manager.slot_tables]
         fields = [("token_ids", B), ("positions", B), ("token_req", B), ("q_start", B + 1), ("kv_len", B),
-                  ("slots", B), ("want_rows", B), ("temperature", B), ("uniform", B)]
+                  ("slots", B), ("token_slots", B), ("want_rows", B), ("temperature", B), ("uniform", B)]
         fields += [(f"table{g}", B * w) for g, w in enumerate(widths)]
         self.spans, at = {}, 0
         for name, n in fields:
@@ -112,6 +112,7 @@ class RecordedDecodeStep:
         tables = [view(f"table{g}").view(B, w) for g, w in enumerate(widths)]
         self.caches = runner.cache_views(tables)
         self.want_rows = view("want_rows")
+        self.token_slots = view("token_slots")  # where the sampler leaves each row's token
         self.temperature = view("temperature").view(torch.float32)
         self.uniform = view("uniform").view(torch.float32)
 
@@ -129,7 +130,7 @@ class RecordedDecodeStep:
 
     def _forward(self):
         logits = self.runner.model.forward(self.ctx, self.caches, self.runner.storage.states, self.want_rows)
-        ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.ctx.slots, self.runner.storage.last_token)
+        ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.token_slots, self.runner.storage.last_token)
         return logits, ids, logprobs
 
     def _fill(self, token_ids, positions, slots, write_slots, temperatures, uniforms) -> None:
@@ -145,7 +146,8 @@ class RecordedDecodeStep:
         put("token_ids", token_ids, 0)
         put("positions", positions, 0)
         put("kv_len", [p + 1 for p in positions], 1)
-        put("slots", write_slots, self.null_slot)
+        put("slots", slots, self.null_slot)
+        put("token_slots", write_slots, self.null_slot)
         at, m = self.spans["token_req"]
         a[at : at + m] = np.arange(m, dtype=np.int32)
         at, m = self.spans["q_start"]
