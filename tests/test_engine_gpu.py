@@ -1,0 +1,191 @@
+"""Generation through the engine's entry points (Python and command line) against
+the plain implementation: greedy and temperature sampling, portions under a token
+budget, finishing, pages that run out, recorded decode steps against eager ones."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_llama
+from tiny_models import CONFIG_A, PAGE_A, PAGE_B, TINY, make_folder, random_tokens
+from tokasaurus_amd import EngineConfig, SamplingParams
+from tokasaurus_amd.engine.engine import Engine
+from tokasaurus_amd.engine.entry import engine_manager
+from tokasaurus_amd.sampling import uniform_for
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_generate(folder, prompt, max_tokens, temperature=0.0, engine_seed=0, request_seed=0, eos=()):
+    """Token by token with the whole sequence recomputed; the same uniform numbers as the engine draws."""
+    cfg, w = plain_llama.load_folder(folder)
+    ids, out, lps = list(prompt), [], []
+    for i in range(max_tokens):
+        logits = plain_llama.forward_logits(cfg, w, ids)[-1]
+        u = uniform_for(engine_seed, request_seed, i) if temperature > 0 else 0.0
+        tok, lp = plain_llama.sample(logits, temperature, u)
+        out.append(tok)
+        lps.append(lp)
+        ids.append(tok)
+        if tok in eos:
+            break
+    return out, lps
+
+
+def engine_for(folders, name, dtype="float32", **kw):
+    _, page = TINY[name]
+    opts = dict(model=str(folders[name]), dtype=dtype, page_size=page, kv_cache_num_tokens=1024,
+                max_seqs_per_forward=8, max_tokens_per_forward=64, allocator_sanity_checks=True)
+    opts.update(kw)
+    return Engine(EngineConfig(**opts))
+
+
+def test_greedy_generation_config_a(folders):
+    """Prompts of 5, 17 and 33 tokens, 8 greedy tokens each, pages of 4."""
+    cfg, _ = TINY["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 40 + n) for n in (5, 17, 33)]
+    engine = engine_for(folders, "A")
+    done = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    for prompt, c in zip(prompts, done):
+        want, want_lp = plain_generate(folders["A"], prompt, 8)
+        assert c.tokens == want and c.finish_reason == "length"
+        assert torch.allclose(torch.tensor(c.logprobs), torch.tensor(want_lp), atol=1e-4)
+    assert engine.runner.manager.num_free_pages() == [1024 // PAGE_A]
+    assert engine.stats.prefill_tokens == 55 and engine.stats.decode_tokens == 3 * 7
+    assert engine.runner.recorded, "decode steps were not recorded"
+
+
+def test_temperature_generation_config_b_in_portions_of_16(folders):
+    """Prompts of 1, 9, 70 and 130 tokens prefilled 16 tokens at a time beside the
+    decoding of the others, then 12 tokens at temperature 0.8, pages of 8."""
+    cfg, _ = TINY["B"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 60 + n) for n in (1, 9, 70, 130)]
+    engine = engine_for(folders, "B", max_prefill_chunk=16, seed=5)
+    params = [SamplingParams(temperature=0.8, max_tokens=12, ignore_eos=True, seed=100 + i) for i in range(4)]
+    done = engine.generate(prompts, params)
+    for i, (prompt, c) in enumerate(zip(prompts, done)):
+        want, want_lp = plain_generate(folders["B"], prompt, 12, temperature=0.8, engine_seed=5, request_seed=100 + i)
+        assert c.tokens == want, (i, c.tokens, want)
+        assert torch.allclose(torch.tensor(c.logprobs), torch.tensor(want_lp), atol=1e-4)
+    assert len(set(tuple(c.tokens) for c in done)) == 4
+    assert engine.stats.steps > 130 // 16
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_bfloat16_generation_follows_the_plain_one(folders, name):
+    cfg, _ = TINY[name]
+    prompts = [random_tokens(n, cfg["vocab_size"], 80 + n) for n in (12, 40)]
+    engine = engine_for(folders, name, dtype="bfloat16")
+    done = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+    pcfg, w = plain_llama.load_folder(folders[name])
+    for prompt, c in zip(prompts, done):
+        # every token the engine chose is, in the plain model given the same history, within
+        # bfloat16 rounding of the best logit (a near tie may fall the other way)
+        ids = list(prompt)
+        for tok in c.tokens:
+            logits = plain_llama.forward_logits(pcfg, w, ids)[-1]
+            assert float(logits.max() - logits[tok]) < 0.08, (tok, int(logits.argmax()))
+            ids.append(tok)
+
+
+def test_recorded_and_eager_decode_steps_agree(folders):
+    """The same requests with and without recorded steps, several replays with eager
+    work (prompt portions of later requests) between them: the same tokens."""
+    cfg, _ = TINY["C"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (30, 8, 55, 21, 40)]
+    results = []
+    for graphs in (True, False):
+        engine = engine_for(folders, "C", dtype="bfloat16", use_hipgraphs=graphs, max_seqs_per_forward=3, max_tokens_per_forward=32)
+        done = engine.generate(prompts, SamplingParams(temperature=0.7, max_tokens=20, ignore_eos=True, seed=3))
+        results.append([(c.tokens, c.logprobs) for c in done])
+        assert bool(engine.runner.recorded) == graphs
+    for (ta, la), (tb, lb) in zip(*results):
+        assert ta == tb
+        assert torch.allclose(torch.tensor(la), torch.tensor(lb), atol=1e-5)
+
+
+def test_finishing_on_an_end_token_and_on_length(folders, tmp_path):
+    cfg, _ = TINY["A"]
+    prompt = random_tokens(9, cfg["vocab_size"], 7)
+    free_run, _ = plain_generate(folders["A"], prompt, 8)
+    eos = free_run[3]
+    first = free_run.index(eos)
+    folder = make_folder(tmp_path / "with_eos", dict(CONFIG_A, eos_token_id=[eos]), seed=11)  # seed of folder A
+    engine = Engine(EngineConfig(model=str(folder), dtype="float32", page_size=PAGE_A, kv_cache_num_tokens=256, max_seqs_per_forward=2))
+    stop, ignore = engine.generate([prompt, prompt], [SamplingParams(max_tokens=8), SamplingParams(max_tokens=8, ignore_eos=True)])
+    assert stop.tokens == free_run[: first + 1] and stop.finish_reason == "stop"
+    assert ignore.tokens == free_run and ignore.finish_reason == "length"
+    one = engine.generate([prompt], SamplingParams(max_tokens=1, ignore_eos=True))[0]  # ends in its prefill step
+    assert one.tokens == free_run[:1] and engine.runner.manager.requests == {}
+
+
+def test_pages_run_out_and_the_newest_request_starts_again(folders):
+    """With admission against the prompt only (the reference's debug option) pages run
+    out while decoding: the newest request is taken out, starts again from its prompt,
+    and every completion is still the plain one."""
+    cfg, _ = TINY["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 20 + n) for n in (14, 15, 13, 16)]
+    engine = engine_for(folders, "A", kv_cache_num_tokens=96, bump_city_population_me=True, max_seqs_per_forward=4)
+    done = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))
+    assert engine.stats.bumps > 0 and sum(c.times_bumped for c in done) == engine.stats.bumps
+    for prompt, c in zip(prompts, done):
+        assert c.tokens == plain_generate(folders["A"], prompt, 20)[0]
+    engine.runner.manager.check()
+    assert engine.runner.manager.num_free_pages() == [96 // PAGE_A]
+    # the default admission reserves a request's whole life: nothing is ever taken out
+    engine = engine_for(folders, "A", kv_cache_num_tokens=96, max_seqs_per_forward=4)
+    again = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))
+    assert engine.stats.bumps == 0 and [c.tokens for c in again] == [c.tokens for c in done]
+    with pytest.raises(ValueError, match="exceeds|more than the whole cache"):
+        engine.submit(random_tokens(90, cfg["vocab_size"], 1), SamplingParams(max_tokens=20))
+
+
+def test_submit_step_abort_and_the_context_manager(folders):
+    cfg, _ = TINY["B"]
+    config = EngineConfig(model=str(folders["B"]), dtype="float32", page_size=PAGE_B, kv_cache_num_tokens=512, max_seqs_per_forward=4)
+    with engine_manager(config) as engine:
+        a = engine.submit(random_tokens(20, cfg["vocab_size"], 1), SamplingParams(max_tokens=50, ignore_eos=True))
+        b = engine.submit(random_tokens(5, cfg["vocab_size"], 2), SamplingParams(max_tokens=4, ignore_eos=True), request_id="mine")
+        assert b == "mine"
+        finished = []
+        for _ in range(3):
+            finished += engine.step()
+        assert engine.abort(a) and not engine.abort("nobody")
+        finished += engine.run_until_done()
+        assert [c.request_id for c in finished] == ["mine"] and len(finished[0].tokens) == 4
+        assert engine.runner.manager.requests == {} and not engine.has_work()
+        with pytest.raises(ValueError, match="outside the vocabulary"):
+            engine.submit([1, cfg["vocab_size"]])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toka_command_line(folders, tmp_path, dtype):
+    """bin/toka key=value ... prints one JSON object a completion."""
+    cfg, page = TINY["B"]
+    prompts = [random_tokens(11, cfg["vocab_size"], 3), random_tokens(4, cfg["vocab_size"], 4)]
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "toka"), f"model={folders['B']}", f"dtype={dtype}", f"page_size={page}",
+         "kv_cache_num_tokens=(8*64)", f"prompt_ids=({json.dumps(prompts)})", "max_tokens=6", "ignore_eos=T", ".eager"],
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.strip()]
+    assert len(lines) == 2 and all(l["finish_reason"] == "length" for l in lines)
+    if dtype == "float32":
+        assert [l["tokens"] for l in lines] == [plain_generate(folders["B"], p, 6)[0] for p in prompts]
+    assert "stats" in proc.stderr
+    # random weights from a config.json alone, and an unknown option refused with the list of known ones
+    model = tmp_path / "fresh"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(CONFIG_A))
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "toka"), f"model={model}", "random_weights=T", "seed=3",
+                           "dtype=float32", "page_size=4", "kv_cache_num_tokens=256", "num_prompts=2", "prompt_len=7", "max_tokens=3"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert (model / "model.safetensors").is_file() and len(proc.stdout.splitlines()) == 2
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "toka"), f"model={model}", "pagesize=4"], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 2 and "unknown option" in proc.stderr and "page_size" in proc.stderr

@@ -10,6 +10,7 @@ top (the reference's forward never returns logits, tokasaurus/model/types.py:403
 
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass
 from pathlib import Path
 
@@ -74,9 +75,12 @@ class RecordedDecodeStep:
     """
 
     def __init__(self, runner: "ModelRunner", size: int):
-        self.runner = runner
+        # no reference to the runner is kept: a runner and its recorded steps must not form a
+        # cycle, or they would be freed by the cyclic collector at a time of its choosing,
+        # possibly while another step is being recorded, when memory must not be released
         self.size = size
         model, storage, manager = runner.model, runner.storage, runner.manager
+        self.model, self.storage, self.manager = model, storage, manager
         device = model.device
         B = size
         widths = [t.shape[1] for t in manager.slot_tables]
@@ -116,21 +120,29 @@ class RecordedDecodeStep:
         self.temperature = view("temperature").view(torch.float32)
         self.uniform = view("uniform").view(torch.float32)
 
-        # once outside the graph (parts plan and allocate what they keep), then recorded
-        stream = torch.cuda.Stream()
-        stream.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(stream):
-            self._forward()
-        torch.cuda.current_stream().wait_stream(stream)
-        torch.cuda.synchronize()
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits, self.ids, self.logprobs = self._forward()
-        torch.cuda.synchronize()
+        # once outside the graph (parts plan and allocate what they keep), then recorded;
+        # the collector stays off meanwhile: nothing may be freed while a graph is recorded
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            stream = torch.cuda.Stream()
+            stream.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(stream):
+                self._forward()
+            torch.cuda.current_stream().wait_stream(stream)
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.logits, self.ids, self.logprobs = self._forward()
+            torch.cuda.synchronize()
+        finally:
+            if was_enabled:
+                gc.enable()
 
     def _forward(self):
-        logits = self.runner.model.forward(self.ctx, self.caches, self.runner.storage.states, self.want_rows)
-        ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.token_slots, self.runner.storage.last_token)
+        logits = self.model.forward(self.ctx, self.caches, self.storage.states, self.want_rows)
+        ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.token_slots, self.storage.last_token)
         return logits, ids, logprobs
 
     def _fill(self, token_ids, positions, slots, write_slots, temperatures, uniforms) -> None:
@@ -162,7 +174,7 @@ class RecordedDecodeStep:
         f[at : at + n] = uniforms
         f[at + n : at + m] = 0.0
         rows = np.asarray(list(slots) + [self.null_slot] * pad, dtype=np.int64)
-        for g, table in enumerate(self.runner.manager.slot_tables):
+        for g, table in enumerate(self.manager.slot_tables):
             at, m = self.spans[f"table{g}"]
             a[at : at + m].reshape(B, table.shape[1])[:] = table[rows]
 
