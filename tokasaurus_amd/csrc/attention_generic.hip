@@ -138,7 +138,7 @@ static void ag_launch(const void* q, int q_stride, void* out, int out_stride, co
                      block_table, table_stride, token_req, positions, nq, nkv, d, P, window, scale);
 }
 
-extern "C" int tk_paged_attention_generic(int dt, const void* q, int q_stride, void* out,
+TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void* out,
                                           int out_stride, const void* kcache, const void* vcache,
                                           const int* block_table, int table_stride,
                                           const int* token_req, const int* positions, int n_tokens,

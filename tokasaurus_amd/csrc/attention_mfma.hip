@@ -340,7 +340,7 @@ static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, hipStream_
 // part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
 // tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when max_splits
 // is 1).  Launches that share scratch must not overlap.
-extern "C" int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
+TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                                        const void* kcache, const void* vcache,
                                        const int* block_table, int table_stride,
                                        const int* q_start, const int* kv_len,

@@ -12,6 +12,9 @@ enum TkDtype { TK_F32 = 0, TK_BF16 = 1 };
 
 typedef __hip_bfloat16 bf16_t;
 
+// Entry points are the only symbols a library exports.
+#define TK_API extern "C" __attribute__((visibility("default")))
+
 // Every entry point returns 0 or a negative code; the text is read with tk_last_error().
 void tk_set_error(const char* fmt, ...);
 

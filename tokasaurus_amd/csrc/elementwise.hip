@@ -4,22 +4,6 @@
 // computes in 32-bit.
 #include "common.h"
 
-#include <stdarg.h>
-#include <stdio.h>
-
-static thread_local char g_error[512];
-
-void tk_set_error(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_error, sizeof(g_error), fmt, ap);
-  va_end(ap);
-}
-
-extern "C" const char* tk_last_error() { return g_error; }
-
-extern "C" int tk_abi_version() { return 9; }
-
 // --------------------------------------------------------------------------
 // embedding: out[t, :] = table[id_t, :]; id_t < 0 names slot -id_t-1 of `last_token`
 // (the token the sampler wrote there in the step before).
@@ -37,7 +21,7 @@ __global__ void embed_gather_kernel(const int* __restrict__ ids, const int* __re
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
 }
 
-extern "C" int tk_embed_gather(int dt, const int* ids, const int* last_token, const void* table,
+TK_API int tk_embed_gather(int dt, const int* ids, const int* last_token, const void* table,
                                void* out, int n_tokens, int hidden, int vocab, hipStream_t stream) {
   TK_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes %d %d %d", n_tokens,
              hidden, vocab);
@@ -77,7 +61,7 @@ __global__ void rmsnorm_kernel(const T* __restrict__ x, const void* __restrict__
   }
 }
 
-extern "C" int tk_rmsnorm(int dt, const void* x, const void* w, int w_f32, void* out, int rows,
+TK_API int tk_rmsnorm(int dt, const void* x, const void* w, int w_f32, void* out, int rows,
                           int hidden, float eps, hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && hidden > 0, "rmsnorm: bad sizes %d %d", rows, hidden);
   if (rows == 0) return 0;
@@ -107,7 +91,7 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   }
 }
 
-extern "C" int tk_swiglu(int dt, const void* gate_up, void* out, int rows, int inter,
+TK_API int tk_swiglu(int dt, const void* gate_up, void* out, int rows, int inter,
                          hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && inter > 0, "swiglu: bad sizes %d %d", rows, inter);
   if (rows == 0) return 0;
@@ -132,7 +116,7 @@ __global__ void gather_rows_kernel(const T* __restrict__ src, int src_stride,
   for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = s[i];
 }
 
-extern "C" int tk_gather_rows(int dt, const void* src, int src_stride, const int* idx, void* out,
+TK_API int tk_gather_rows(int dt, const void* src, int src_stride, const int* idx, void* out,
                               int n, int width, hipStream_t stream) {
   TK_REQUIRE(n >= 0 && width > 0 && src_stride >= width, "gather_rows: bad sizes %d %d %d", n,
              width, src_stride);
@@ -160,7 +144,7 @@ __global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __r
   sin_t[i] = sinf(angle);
 }
 
-extern "C" int tk_rope_table(const float* inv_freq, float* cos_t, float* sin_t, int n_pos, int half,
+TK_API int tk_rope_table(const float* inv_freq, float* cos_t, float* sin_t, int n_pos, int half,
                              hipStream_t stream) {
   TK_REQUIRE(n_pos > 0 && half > 0, "rope_table: bad sizes %d %d", n_pos, half);
   const long total = (long)n_pos * half;
@@ -223,7 +207,7 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
   }
 }
 
-extern "C" int tk_rope_append(int dt, void* qkv, int row_stride, const int* positions,
+TK_API int tk_rope_append(int dt, void* qkv, int row_stride, const int* positions,
                               const int* token_req, const int* block_table, int table_stride,
                               const float* cos_t, const float* sin_t, void* kcache, void* vcache,
                               int n_tokens, int nq, int nkv, int d, int P, int write_cache,
@@ -255,11 +239,35 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n) {
   if (i < n) p[i] = v;
 }
 
-extern "C" int tk_fill_u32(void* p, uint32_t value, size_t n, hipStream_t stream) {
+TK_API int tk_fill_u32(void* p, uint32_t value, size_t n, hipStream_t stream) {
   if (n == 0) return 0;
   TK_REQUIRE(n < ((size_t)1 << 40), "fill: too many elements");
   hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
                      (uint32_t*)p, value, n);
   TK_CHECK_LAUNCH("fill_u32");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// add: out = x + y, both rounded operands added in 32-bit and rounded once (the residual
+// sum behind a product that a library computed)
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rows_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<T>(to_f32<T>(x[i]) + to_f32<T>(y[i]));
+}
+
+TK_API int tk_add(int dt, const void* x, const void* y, void* out, size_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  TK_REQUIRE(n < ((size_t)1 << 40), "add: too many elements");
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dt == TK_F32)
+    hipLaunchKernelGGL(add_rows_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x,
+                       (const float*)y, (float*)out, n);
+  else
+    hipLaunchKernelGGL(add_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)x,
+                       (const bf16_t*)y, (bf16_t*)out, n);
+  TK_CHECK_LAUNCH("add");
   return 0;
 }

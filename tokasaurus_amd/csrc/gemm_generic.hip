@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 }
 
 // out_f32: write C as 32-bit floats whatever the storage type (the logits).
-extern "C" int tk_gemm_generic(int dt, const void* A, int lda, const void* W, void* C, int ldc,
+TK_API int tk_gemm_generic(int dt, const void* A, int lda, const void* W, void* C, int ldc,
                                const void* residual, int ldr, int M, int N, int K, int out_f32,
                                hipStream_t stream) {
   TK_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K && ldc >= N, "gemm_generic: bad sizes M=%d N=%d K=%d lda=%d ldc=%d",

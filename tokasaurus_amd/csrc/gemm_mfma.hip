@@ -524,7 +524,7 @@ static bool launch_mb(const GemmArgs& a, int epi, bool norm, int NT, int groups,
 // K inside a workgroup (0 = choose); tiles: weight tiles of 16 rows per wavefront, 1 or 2
 // (0 = choose; SwiGLU always pairs gate and up); staged: -1 = choose, 0 = skinny, 1 = staged;
 // tile_rows: weight rows of a tile that the skinny kernel uses, 16 or 8 (0 = choose).
-extern "C" int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, int ldc,
+TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, int ldc,
                                    const void* residual, int ldr, const void* norm_w,
                                    int norm_w_f32, float eps, int M, int N, int K, int epi,
                                    int waves_k, int tiles, int staged, int tile_rows,
@@ -601,29 +601,5 @@ extern "C" int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* 
   }
   TK_REQUIRE(ok, "gemm_skinny: the kernel's local memory could not be reserved");
   TK_CHECK_LAUNCH("gemm_skinny");
-  return 0;
-}
-
-// --------------------------------------------------------------------------
-// Epilogue for products that a library computed (many rows, prefill):
-//   out = x + y, both rounded operands added in 32-bit and rounded once
-// --------------------------------------------------------------------------
-template <typename T>
-__global__ void add_rows_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ out, size_t n) {
-  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) out[i] = from_f32<T>(to_f32<T>(x[i]) + to_f32<T>(y[i]));
-}
-
-extern "C" int tk_add(int dt, const void* x, const void* y, void* out, size_t n, hipStream_t stream) {
-  if (n == 0) return 0;
-  TK_REQUIRE(n < ((size_t)1 << 40), "add: too many elements");
-  const unsigned blocks = (unsigned)((n + 255) / 256);
-  if (dt == TK_F32)
-    hipLaunchKernelGGL(add_rows_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x,
-                       (const float*)y, (float*)out, n);
-  else
-    hipLaunchKernelGGL(add_rows_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)x,
-                       (const bf16_t*)y, (bf16_t*)out, n);
-  TK_CHECK_LAUNCH("add");
   return 0;
 }

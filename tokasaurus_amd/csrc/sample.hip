@@ -171,10 +171,10 @@ __global__ __launch_bounds__(SM_THREADS) void sample_finish_kernel(
   }
 }
 
-extern "C" int tk_sample_chunks(int vocab) { return (vocab + SM_CHUNK - 1) / SM_CHUNK; }
+TK_API int tk_sample_chunks(int vocab) { return (vocab + SM_CHUNK - 1) / SM_CHUNK; }
 
 // part_max, part_sum (float) and part_arg (int) hold rows * tk_sample_chunks(vocab) entries each.
-extern "C" int tk_sample(const float* logits, int ld, int rows, int vocab, const float* temperature,
+TK_API int tk_sample(const float* logits, int ld, int rows, int vocab, const float* temperature,
                          const float* uniform, const int* slots, int* last_token, int* out_ids,
                          float* out_logprobs, float* part_max, float* part_sum, int* part_arg,
                          hipStream_t stream) {

@@ -1,10 +1,14 @@
-"""Builds the gfx950 kernel library from ``tokasaurus_amd/csrc`` with hipcc.
+"""Builds the gfx950 kernel libraries from ``tokasaurus_amd/csrc`` with hipcc.
 
-The library is one shared object loaded through ctypes (no Python headers, no
-torch headers), so a fresh checkout builds it in well under a minute and any
-user who can write the build folder can do so.  ``ensure_built`` is what the
-loader calls: it compiles only when no library matching the current sources
-exists, and prints a line per file meanwhile.
+There are two shared objects, loaded through ctypes (no Python headers, no torch
+headers): ``core`` holds the kernels every model needs in either storage type,
+``mfma`` the bfloat16 matrix-core kernels, which a 32-bit run never loads and so
+never compiles.  A fresh checkout builds what it needs at its first call in
+well under a minute.  ``ensure_built`` is what the loader calls: it compiles only
+when no library matching the current sources exists, and prints a line per file
+meanwhile.  The libraries live in ``tokasaurus_amd/kernels/_build``; when that
+folder cannot be written (a checkout owned by someone else) they are built in a
+folder of the user's own under the system's temporary folder.
 """
 
 from __future__ import annotations
@@ -14,18 +18,23 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 import time
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
-BUILD_DIR = Path(__file__).resolve().parent / "_build"
-LIB_NAME = "libtokasaurus_hip.so"
+IN_TREE_DIR = Path(__file__).resolve().parent / "_build"
+GROUPS = {
+    "core": ["errors.hip", "elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sample.hip"],
+    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip"],
+}
 
 ARCH = "gfx950"
 # packed 32-bit float instructions are kept off for every kernel of this library
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}",
+    "-fvisibility=hidden",
     "-O3",
     "-fPIC",
     "-std=c++17",
@@ -41,8 +50,8 @@ class BuildError(RuntimeError):
     pass
 
 
-def sources() -> list[Path]:
-    return sorted(CSRC.glob("*.hip"))
+def sources(group: str) -> list[Path]:
+    return [CSRC / name for name in GROUPS[group]]
 
 
 def _hipcc() -> str:
@@ -52,23 +61,51 @@ def _hipcc() -> str:
     return exe
 
 
-def _digest() -> str:
+def _digest(group: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for p in sorted(CSRC.glob("*")):
-        if p.suffix in (".hip", ".h"):
-            h.update(p.name.encode())
-            h.update(p.read_bytes())
+    for p in sorted(CSRC.glob("*.h")) + sources(group):
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
     return h.hexdigest()
 
 
-def library_path() -> Path:
-    return BUILD_DIR / LIB_NAME
+def _writable(folder: Path) -> bool:
+    try:
+        folder.mkdir(parents=True, exist_ok=True)
+        probe = folder / f".probe{os.getpid()}"
+        probe.write_text("")
+        probe.unlink()
+        return True
+    except OSError:
+        return False
 
 
-def is_current() -> bool:
-    stamp = BUILD_DIR / "stamp"
-    return library_path().is_file() and stamp.is_file() and stamp.read_text().strip() == _digest()
+def build_dir() -> Path:
+    """The in-tree folder, or a folder of the user's own when that one cannot be written."""
+    if _writable(IN_TREE_DIR):
+        return IN_TREE_DIR
+    own = Path(tempfile.gettempdir()) / f"tokasaurus_amd_build_{os.getuid()}"
+    if not _writable(own):
+        raise BuildError(f"neither {IN_TREE_DIR} nor {own} can be written: nowhere to build the kernel library")
+    return own
+
+
+def library_name(group: str) -> str:
+    return f"libtokasaurus_{group}.so"
+
+
+def find_current(group: str) -> Path | None:
+    """A library of this group built from the current sources, wherever it was built."""
+    digest = _digest(group)
+    for folder in (IN_TREE_DIR, Path(tempfile.gettempdir()) / f"tokasaurus_amd_build_{os.getuid()}"):
+        lib, stamp = folder / library_name(group), folder / f"stamp_{group}"
+        try:
+            if lib.is_file() and stamp.is_file() and stamp.read_text().strip() == digest:
+                return lib
+        except OSError:
+            continue
+    return None
 
 
 def _say(msg: str) -> None:
@@ -84,43 +121,58 @@ def _compile_one(hipcc: str, src: Path, obj: Path) -> tuple[Path, float]:
     return src, time.time() - t0
 
 
-def build(force: bool = True, jobs: int | None = None) -> Path:
-    """Compile every source and link the library.  ``force=False`` returns at
-    once when a library built from the current sources is already there."""
-    if not force and is_current():
-        return library_path()
+def build_group(group: str, jobs: int | None = None) -> Path:
+    """Compile the sources of one group and link its library."""
     hipcc = _hipcc()
-    BUILD_DIR.mkdir(parents=True, exist_ok=True)
-    srcs = sources()
-    if not srcs:
-        raise BuildError(f"no kernel sources under {CSRC}")
+    folder = build_dir()
+    srcs = sources(group)
+    missing = [s.name for s in srcs if not s.is_file()]
+    if missing:
+        raise BuildError(f"kernel sources missing under {CSRC}: {missing}")
     jobs = jobs or min(len(srcs), int(os.environ.get("MAX_JOBS", "8")), 16)
-    _say(f"compiling {len(srcs)} HIP sources for {ARCH} with {jobs} jobs")
-    objs = [BUILD_DIR / (s.stem + ".o") for s in srcs]
+    _say(f"compiling the {group} kernels ({len(srcs)} HIP sources) for {ARCH} with {jobs} jobs into {folder}")
+    objs = [folder / (f"{group}_{s.stem}.{os.getpid()}.o") for s in srcs]
     t0 = time.time()
-    with ThreadPoolExecutor(max_workers=jobs) as pool:
-        futures = [pool.submit(_compile_one, hipcc, s, o) for s, o in zip(srcs, objs)]
-        for fut in futures:
-            src, dt = fut.result()
-            _say(f"  {src.name} done in {dt:.1f}s")
-    tmp = BUILD_DIR / (LIB_NAME + f".tmp{os.getpid()}")
-    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
-    proc = subprocess.run(link, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise BuildError(f"link failed:\n{proc.stderr[-4000:]}")
-    os.replace(tmp, library_path())
-    (BUILD_DIR / "stamp").write_text(_digest() + "\n")
-    _say(f"built {library_path()} in {time.time() - t0:.1f}s")
-    return library_path()
+    try:
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            futures = [pool.submit(_compile_one, hipcc, s, o) for s, o in zip(srcs, objs)]
+            for fut in futures:
+                src, dt = fut.result()
+                _say(f"  {src.name} done in {dt:.1f}s")
+        tmp = folder / (library_name(group) + f".tmp{os.getpid()}")
+        link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
+        proc = subprocess.run(link, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise BuildError(f"link failed:\n{proc.stderr[-4000:]}")
+        os.replace(tmp, folder / library_name(group))
+        (folder / f"stamp_{group}").write_text(_digest(group) + "\n")
+    finally:
+        for o in objs:
+            try:
+                o.unlink()
+            except OSError:
+                pass
+    _say(f"built {folder / library_name(group)} in {time.time() - t0:.1f}s")
+    return folder / library_name(group)
 
 
-def ensure_built() -> Path:
-    """The library for the current sources, compiling it if it is not there."""
-    if is_current():
-        return library_path()
-    if library_path().is_file():
-        _say("the built library does not match the sources; building again")
-    return build(force=True)
+def build(force: bool = True) -> list[Path]:
+    """Every group.  ``force=False`` skips a group whose library matches the current sources."""
+    out = []
+    for group in GROUPS:
+        current = None if force else find_current(group)
+        out.append(current or build_group(group))
+    return out
+
+
+def ensure_built(group: str) -> Path:
+    """The library of a group for the current sources, compiling it if it is not there."""
+    current = find_current(group)
+    if current is not None:
+        return current
+    if (IN_TREE_DIR / library_name(group)).is_file():
+        _say(f"the built {group} library does not match the sources; building again")
+    return build_group(group)
 
 
 if __name__ == "__main__":

@@ -451,7 +451,7 @@ def sample(
         _need(slots.numel() == rows, "sample: one slot a row")
     ids = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     logprobs = torch.empty((rows,), dtype=torch.float32, device=logits.device) if want_logprobs else None
-    chunks = load().tk_sample_chunks(vocab)
+    chunks = load("core").tk_sample_chunks(vocab)
     part = torch.empty((3, max(rows, 1) * chunks), dtype=torch.float32, device=logits.device)
     call(
         "tk_sample",
