@@ -163,7 +163,7 @@ GEMM_SHAPES = [(2048, 256), (1000, 96), (777, 264), (48, 2048), (16, 32), (3072,
 
 @pytest.mark.parametrize("m", [1, 5, 16, 17, 40, 64, 100, 128])
 @pytest.mark.parametrize("shape", GEMM_SHAPES)
-@pytest.mark.parametrize("mode", ["store", "residual", "f32", "swiglu", "norm_store", "norm_swiglu", "norm_f32_weight32"])
+@pytest.mark.parametrize("mode", ["store", "residual", "f32", "swiglu"])
 def test_gemm_skinny(m, shape, mode):
     from tokasaurus_amd.kernels import ops
 
@@ -182,11 +182,6 @@ def test_gemm_skinny(m, shape, mode):
         kwargs["swiglu"] = ref_kwargs["swiglu"] = True
     if "f32" in mode:
         kwargs["out_f32"] = True
-    if "norm" in mode:
-        nw = 1.0 + 0.1 * torch.randn((k,), generator=g)
-        nw = nw if mode.endswith("weight32") else nw.to(torch.bfloat16)
-        kwargs.update(norm_weight=nw.cuda(), norm_eps=1e-5)
-        ref_kwargs.update(norm_weight=nw, eps=1e-5)
     ref = gemm_reference(a, w, **ref_kwargs)
     for staged, tile_rows in ((0, 16), (0, 8), (1, 0)) if m > 16 else ((0, 16), (0, 8)):
         got = ops.gemm_skinny_bf16(a.cuda(), w.cuda(), staged=staged, tile_rows=tile_rows, **kwargs).float().cpu()
@@ -194,11 +189,78 @@ def test_gemm_skinny(m, shape, mode):
         # 32-bit accumulation; a bfloat16 result is rounded to 8 bits, and a rounding of an
         # intermediate (norm, gate, up) may fall the other way than in the reference
         tol = dict(atol=2e-5, rtol=2e-5) if mode == "f32" else dict(atol=3e-2, rtol=2e-2)
-        if mode == "norm_f32_weight32":
-            tol = dict(atol=1e-2, rtol=1e-2)  # 32-bit output of a product of once-rounded inputs
         err = (got - ref).abs()
         bad = err > tol["atol"] + tol["rtol"] * ref.abs()
         assert not bad.any(), f"staged={staged} tile_rows={tile_rows}: {int(bad.sum())} wrong, largest error {float(err.max()):.3e}"
+
+
+@pytest.mark.parametrize("m", [1, 7, 16, 40, 128])
+@pytest.mark.parametrize("weight32", [False, True])
+def test_gemm_norm_between_two_products(m, weight32):
+    """The residual epilogue leaves x * w and partial sums of x^2 for the norm that follows;
+    the next product divides its rows by their rms: together RMSNorm(x) W^T without a norm kernel."""
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(m)
+    hidden, inter, n2 = 200, 96, 1000
+    a = torch.randn((m, inter), generator=g).to(torch.bfloat16)
+    w1 = (torch.randn((hidden, inter), generator=g) / math.sqrt(inter)).to(torch.bfloat16)
+    res = (torch.randn((m, hidden), generator=g) * 2).to(torch.bfloat16)
+    nw = 1.0 + 0.1 * torch.randn((hidden,), generator=g)
+    nw = nw if weight32 else nw.to(torch.bfloat16)
+    w2 = (torch.randn((n2, hidden), generator=g) / math.sqrt(hidden)).to(torch.bfloat16)
+    for tile_rows in (8, 16):
+        x, pre = ops.gemm_skinny_bf16(a.cuda(), w1.cuda(), residual=res.cuda(), emit_weight=nw.cuda(), tile_rows=tile_rows)
+        x_ref = gemm_reference(a, w1, residual=res)
+        assert torch.allclose(x.cpu().float(), x_ref, atol=3e-2, rtol=2e-2)
+        xr = x.cpu().float()  # what the engine holds: the rounded rows
+        assert tuple(pre.sumsq.shape) == (m, -(-hidden // tile_rows))
+        assert torch.allclose(pre.sumsq.sum(-1).cpu(), xr.pow(2).sum(-1), rtol=1e-5)
+        assert torch.allclose(pre.scaled.cpu().float(), (nw.float() * xr).to(torch.bfloat16).float(), atol=1e-6, rtol=1e-2)
+        want = gemm_reference(x.cpu(), w2, norm_weight=nw, eps=1e-5)
+        for staged in (0, 1):
+            for out_f32 in (False, True):
+                got = ops.gemm_skinny_bf16(pre.scaled, w2.cuda(), prenorm=pre, norm_eps=1e-5, out_f32=out_f32, staged=staged)
+                assert torch.allclose(got.cpu().float(), want, atol=3e-2, rtol=2e-2), (tile_rows, staged, out_f32)
+        gu = torch.cat([w2[:500], w2[500:]])  # gate over up
+        got = ops.gemm_skinny_bf16(pre.scaled, gu.cuda(), prenorm=pre, norm_eps=1e-5, swiglu=True)
+        want_g, want_u = bf16_round(want[:, :500]), bf16_round(want[:, 500:])
+        assert torch.allclose(got.cpu().float(), bf16_round(torch.nn.functional.silu(want_g)) * want_u, atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("m", [1, 9, 16, 33, 128])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 2, 64, 16), (6, 2, 48, 16), (2, 2, 128, 16)])
+def test_gemm_rotation_with_append_epilogue(m, shape):
+    """The [q | k | v] product with rotation and append in its epilogue leaves the same
+    queries and the same pages as the plain product followed by the rotation kernel."""
+    from tokasaurus_amd.kernels import ops
+
+    nq, nkv, d, page = shape
+    hidden = 96
+    g = torch.Generator().manual_seed(m + d)
+    a = torch.randn((m, hidden), generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(((nq + 2 * nkv) * d, hidden), generator=g) / math.sqrt(hidden)).to(torch.bfloat16).cuda()
+    # every row is a request of its own at some position (a decode batch), pages shuffled
+    positions = torch.randint(0, 90, (m,), generator=g).to(torch.int32)
+    width = -(-90 // page)
+    table = torch.randperm(m * width, generator=g).to(torch.int32).view(m, width)
+    token_req = torch.arange(m, dtype=torch.int32)
+    inv = torch.arange(0, d, 2).float() / d
+    cos = torch.cos(torch.arange(100)[:, None] * (10000.0 ** -inv)[None, :]).contiguous().cuda()
+    sin = torch.sin(torch.arange(100)[:, None] * (10000.0 ** -inv)[None, :]).contiguous().cuda()
+    caches = []
+    for fused in (False, True):
+        kc = torch.full((m * width, nkv, page, d), 7.0, dtype=torch.bfloat16).cuda()
+        vc = torch.full((m * width, nkv, d, page), 7.0, dtype=torch.bfloat16).cuda()
+        if fused:
+            for tile_rows in (8, 16):
+                rope = ops.RopeAppend(positions.cuda(), token_req.cuda(), table.cuda(), cos, sin, kc, vc, nq, nkv, d, page)
+                q = ops.gemm_skinny_bf16(a, w, rope=rope, tile_rows=tile_rows)
+                assert torch.equal(q, caches[0][0]) and torch.equal(kc, caches[0][1]) and torch.equal(vc, caches[0][2]), tile_rows
+        else:
+            qkv = ops.gemm_skinny_bf16(a, w)
+            ops.rope_append(qkv, positions.cuda(), token_req.cuda(), table.cuda(), cos, sin, kc, vc, nq, nkv, d, page)
+            caches.append((qkv[:, : nq * d].contiguous(), kc, vc))
 
 
 def test_gemm_rows_do_not_depend_on_the_batch():

@@ -19,6 +19,7 @@ from tiny_models import CONFIG_A, CONFIG_B, random_tokens
 from tokasaurus_amd.engine.batch import PlannedEntry, layout, to_device
 from tokasaurus_amd.engine.runner import ModelRunner
 from tokasaurus_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, PartSpec
+from tokasaurus_amd.parts.block import stream_and_prepared
 from tokasaurus_amd.parts.embedding import LMHead, TokenEmbedding
 from tokasaurus_amd.parts.linear import Placer
 from tokasaurus_amd.weights import write_random_model
@@ -71,7 +72,8 @@ def test_norm_feed_forward_embedding_and_head_alone(dtype):
     res = rand((11, H), g, dt)
     gate, up = xf @ f32["g.weight"].T, xf @ f32["u.weight"].T
     want = res.float() + (torch.nn.functional.silu(gate) * up) @ f32["d.weight"].T
-    assert torch.allclose(ff.forward(x.cuda(), res.cuda()).cpu().float(), want, **PART_TOL[dtype])
+    got, _ = stream_and_prepared(ff.forward(x.cuda(), res.cuda()))
+    assert torch.allclose(got.cpu().float(), want, **PART_TOL[dtype])
 
     emb = TokenEmbedding(V, H, "e.weight")
     emb.load(tensors, placer)
@@ -153,9 +155,9 @@ def test_attention_mixer_and_block_alone(dtype, shape):
             cache = CacheView(keys, values, table, page)
             x = torch.cat([xs[r][s : s + n] for r, s, n in zip(reqs, starts, q_lens)]).cuda()
             if part == "mixer":
-                out = built.forward(x, x, ctx, cache, None, None)  # h = residual = x
+                out, _ = stream_and_prepared(built.forward(x, x, ctx, cache, None, None))  # h = residual = x
             else:
-                out = built.forward(x, ctx, cache, None, None)
+                out, _ = stream_and_prepared(built.forward(x, ctx, cache, None, None))
             at = 0
             for r, s, n in zip(reqs, starts, q_lens):
                 got.setdefault(r, []).append(out[at : at + n].cpu().float())

@@ -19,19 +19,23 @@
 //     part of A passes through LDS (double buffered, 4 steps of 32 a round) so that A
 //     is read from the caches once per workgroup and not once per wavefront.
 //
-// Norm in front (norm_w != null): the product of RMSNorm(A) is rstd[row] * ((A * w) W^T),
-// so the kernel multiplies A by the norm weight on the way in (rounded to bfloat16
-// once), sums the squares of the A values it reads anyway in 32-bit, and scales each
-// output row by rstd = 1 / sqrt(mean(A^2) + eps) in the epilogue: no pass over A of its
-// own and no wait in front of the weight stream.  Epilogues: plain store, + residual,
+// Norm in front (sumsq_in != null).  The product of RMSNorm(x) is rstd[row] * ((x * w) W^T).
+// The kernel that produced x (the residual epilogue below, when emit_w is given) has
+// already written A = x * w, rounded once, and for every row the sum of x^2 over each
+// of its tiles; this kernel adds those partial sums in tile order and scales its output
+// rows by rstd = 1 / sqrt(sum / K + eps) in the epilogue.  So a norm between two
+// products costs no kernel and no pass over the row of its own.
+// Epilogues: plain store, + residual (optionally emitting what the next norm needs),
 // SwiGLU (the wavefront takes the same 16 rows of the gate and of the up projection),
-// 32-bit store.
+// 32-bit store, and rotation with append: the output rows are [q heads | k heads |
+// v heads]; a workgroup takes the rows (c, c + d/2) of a head together, rotates q and k
+// by the token's position, writes q to the output and k and v into the token's page.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_F32 = 3 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_F32 = 3, EPI_ROPE = 4 };
 
 struct GemmArgs {
   const bf16_t* A;
@@ -41,9 +45,28 @@ struct GemmArgs {
   int ldc;
   const bf16_t* residual;
   int ldr;
-  const void* norm_w;  // [K] bfloat16, or float when norm_w_f32
-  int norm_w_f32;
+  // norm in front: per row `parts_in` partial sums of squares of the un-normed row
+  const float* sumsq_in;
+  int parts_in;
   float eps;
+  // residual epilogue, for the norm that follows: weight [N] (bfloat16, or float when
+  // emit_w_f32), x * w rounded once [M, N], and per row one partial sum of x^2 a tile
+  const void* emit_w;
+  int emit_w_f32;
+  bf16_t* emit_scaled;
+  int ld_emit;
+  float* emit_sumsq;
+  int parts_out;
+  // rotation with append
+  const int* positions;
+  const int* token_req;
+  const int* block_table;
+  int table_stride;
+  const float* cos_t;  // [positions][d / 2], null: no rotation
+  const float* sin_t;
+  bf16_t* kcache;  // [page][kv head][P][d]
+  bf16_t* vcache;  // [page][kv head][d][P]
+  int nq, nkv, d, P;
   int M, N, K;  // N: outputs (for SwiGLU the intermediate size; W then has 2N rows, gate first)
   int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
 };
@@ -96,36 +119,115 @@ __device__ __forceinline__ bf16x8_t zero8() {
   return z;
 }
 
-// 8 values of a row times the norm weight, rounded once; their squares are added to `ss`.
-__device__ __forceinline__ bf16x8_t weigh_piece(bf16x8_t x, const void* w, int w_f32, int k, float& ss) {
-  bf16x8_t o;
-  if (w_f32) {
-    const float* wf = (const float*)w + k;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float xe = (float)x[e];
-      ss = fmaf(xe, xe, ss);
-      o[e] = (__bf16)(wf[e] * xe);
+// 1 / rms of every row of A from the partial sums its producer left, into LDS `scale`
+// (16 * MB floats).  A wavefront takes a row at a time: every lane adds 4 parts (one
+// 16-byte load), then the lanes' sums are added by a butterfly, so the order is fixed.
+template <int MB>
+__device__ __forceinline__ void row_scales(const GemmArgs& a, float* scale) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int nwaves = blockDim.x >> 6;
+  const int rows = min(a.M, 16 * MB);
+  const bool vec = (a.parts_in & 3) == 0;
+  for (int token = wave; token < rows; token += nwaves) {
+    const float* part = a.sumsq_in + (size_t)token * a.parts_in;
+    float ss = 0.f;
+    for (int p = lane * 4; p < a.parts_in; p += 256) {
+      if (vec) {
+        const f32x4_t v = *(const f32x4_t*)(part + p);
+        ss += (v[0] + v[1]) + (v[2] + v[3]);
+      } else {
+        for (int j = 0; j < 4 && p + j < a.parts_in; ++j) ss += part[p + j];
+      }
     }
-  } else {
-    const bf16x8_t wv = *(const bf16x8_t*)((const bf16_t*)w + k);
+    ss = wave_sum(ss);
+    if (lane == 0) scale[token] = 1.0f / sqrtf(ss / (float)a.K + a.eps);
+  }
+}
+
+// The residual epilogue's extra outputs for the norm that follows: x * w rounded once,
+// and the sum of x^2 over this tile's columns.  All 64 lanes of a wavefront call this
+// together; lanes (token, qq = 0..3) share a token.
+__device__ __forceinline__ void emit_for_norm(const GemmArgs& a, const float (&x)[4], bool live, int token,
+                                              int n, int part, int lane) {
+  float ss = 0.f;
+  if (live) {
+    bf16_t* dst = a.emit_scaled + (size_t)token * a.ld_emit + n;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float xe = (float)x[e];
-      ss = fmaf(xe, xe, ss);
-      o[e] = (__bf16)((float)wv[e] * xe);
+    for (int j = 0; j < 4; ++j) {
+      if (n + j < a.N) {
+        const float xr = round_to<bf16_t>(x[j]);
+        const float w = a.emit_w_f32 ? ((const float*)a.emit_w)[n + j] : __bfloat162float(((const bf16_t*)a.emit_w)[n + j]);
+        ss = fmaf(xr, xr, ss);
+        dst[j] = __float2bfloat16(w * xr);
+      }
     }
   }
-  return o;
+  const float s1 = __shfl_xor(ss, 16, 64);
+  const float lo = (lane & 16) ? s1 + ss : ss + s1;
+  const float s2 = __shfl_xor(lo, 32, 64);
+  const float total = (lane & 32) ? s2 + lo : lo + s2;
+  if (live && (lane >> 4) == 0) a.emit_sumsq[(size_t)token * a.parts_out + part] = total;
+}
+
+// Rotation with append for 4 columns c .. c+3 of head h (and their partners c + d/2): x1, x2
+// are the products rounded to bfloat16 as a plain store would leave them.
+__device__ __forceinline__ void rope_store(const GemmArgs& a, f32x4_t s0, f32x4_t s1, int token, int h, int c) {
+  if (token >= a.M) return;
+  const int half = a.d >> 1;
+  const int pos = a.positions[token];
+  float o1[4], o2[4];
+  const bool rotate = h < a.nq + a.nkv && a.cos_t != nullptr;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float x1 = round_to<bf16_t>(s0[j]), x2 = round_to<bf16_t>(s1[j]);
+    if (rotate && c + j < half) {
+      const float cj = a.cos_t[(size_t)pos * half + c + j], sj = a.sin_t[(size_t)pos * half + c + j];
+      o1[j] = x1 * cj - x2 * sj;
+      o2[j] = x2 * cj + x1 * sj;
+    } else {
+      o1[j] = x1;
+      o2[j] = x2;
+    }
+  }
+  if (h < a.nq) {
+    bf16_t* dst = (bf16_t*)a.C + (size_t)token * a.ldc + (size_t)h * a.d + c;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (c + j < half) {
+        dst[j] = __float2bfloat16(o1[j]);
+        dst[j + half] = __float2bfloat16(o2[j]);
+      }
+    return;
+  }
+  const int page = a.block_table[(size_t)a.token_req[token] * a.table_stride + pos / a.P];
+  const int off = pos % a.P;
+  if (h < a.nq + a.nkv) {
+    bf16_t* dst = a.kcache + (((size_t)page * a.nkv + (h - a.nq)) * a.P + off) * a.d + c;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (c + j < half) {
+        dst[j] = __float2bfloat16(o1[j]);
+        dst[j + half] = __float2bfloat16(o2[j]);
+      }
+  } else {
+    bf16_t* dst = a.vcache + (((size_t)page * a.nkv + (h - a.nq - a.nkv)) * a.d + c) * a.P + off;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (c + j < half) {
+        dst[(size_t)j * a.P] = __float2bfloat16(o1[j]);
+        dst[(size_t)(j + half) * a.P] = __float2bfloat16(o2[j]);
+      }
+  }
 }
 
 #define SK_MAX_WAVES 16
 
-// LDS of the skinny kernel: [sums: waves * NT * MB * 64 f32x4][squares: waves * 16 * MB floats]
+// LDS of the skinny kernel: [scales: 16 * MB floats when NORM][sums: waves * NT * MB * 64 f32x4]
 template <int MB, int NT, int EPI, bool NORM>
 __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int U = (NT + MB <= 3) ? 8 : ((NT + MB <= 6) ? 4 : 2);  // steps whose loads are in flight together
+  constexpr bool PAIRED = EPI == EPI_SWIGLU || EPI == EPI_ROPE;     // two tiles that meet in the epilogue
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int WK = blockDim.x >> 6;
   const int r = lane & 15, q = lane >> 4;
@@ -133,19 +235,26 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
   const int K32 = (a.K + 31) >> 5;
   const int ks0 = (int)((long)K32 * wave / WK), ks1 = (int)((long)K32 * (wave + 1) / WK);
   const bool k_exact = (a.K & 31) == 0;
-  f32x4_t* red = (f32x4_t*)smem;
-  float* sq = (float*)(red + (WK > 1 ? (size_t)WK * NT * MB * 64 : 0));
+  float* scales = (float*)smem;
+  f32x4_t* red = (f32x4_t*)(smem + (NORM ? 16 * MB * sizeof(float) : 0));
+  if (NORM) row_scales<MB>(a, scales);
 
   // rows of W this lane streams (clamped: rows past the end are masked at the store);
   // with tiles of 8 rows the upper lanes have no row and hold zeros
   const int TH = a.TH;
   const bool has_row = r < TH;
+  int rope_head = 0, rope_col = 0;  // EPI_ROPE: the head and the first column of this workgroup's pair of tiles
   const bf16_t* wp[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     int row;
     if (EPI == EPI_SWIGLU) {
       row = min(g * TH + r, a.N - 1) + t * a.N;  // t = 0 gate, t = 1 up
+    } else if (EPI == EPI_ROPE) {
+      const int pairs = (a.d / 2 + TH - 1) / TH;  // pairs of tiles a head
+      rope_head = g / pairs;
+      rope_col = (g - rope_head * pairs) * TH;
+      row = rope_head * a.d + min(rope_col + r, a.d / 2 - 1) + t * (a.d / 2);
     } else {
       row = min((g * NT + t) * TH + r, a.N - 1);
     }
@@ -154,10 +263,6 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
   const bf16_t* ap[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) ap[mb] = a.A + (size_t)min(mb * 16 + r, a.M - 1) * a.lda + q * 8;
-
-  float ss[MB];  // squares of the values of row 16 mb + r that this lane has read
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) ss[mb] = 0.f;
 
   f32x4_t acc[NT][MB];
 #pragma unroll
@@ -182,13 +287,6 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) av[u][mb] = *(const bf16x8_t*)(ap[mb] + (size_t)(ks + u) * 32);
       }
-      if (NORM) {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            av[u][mb] = weigh_piece(av[u][mb], a.norm_w, a.norm_w_f32, (ks + u) * 32 + q * 8, ss[mb]);
-      }
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -209,10 +307,7 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
       if (!k_ok || !has_row) w[t] = zero8();
     }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      av[mb] = *(const bf16x8_t*)(ap[mb] + off);
-      if (NORM && k_ok) av[mb] = weigh_piece(av[mb], a.norm_w, a.norm_w_f32, ks * 32 + q * 8, ss[mb]);
-    }
+    for (int mb = 0; mb < MB; ++mb) av[mb] = *(const bf16x8_t*)(ap[mb] + off);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -220,37 +315,23 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
         acc[t][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t], av[mb], acc[t][mb], 0, 0, 0);
   }
 
-  if (NORM) {
-    // the row's squares over this wavefront's part of K: every lane of the row gets the sum
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      ss[mb] += __shfl_xor(ss[mb], 16, 64);
-      ss[mb] += __shfl_xor(ss[mb], 32, 64);
-    }
-  }
   // add the wavefronts' partial sums in wavefront order
   if (WK > 1) {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) red[(wave * NT * MB + t * MB + mb) * 64 + lane] = acc[t][mb];
-    if (NORM && q == 0) {
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) sq[wave * 16 * MB + mb * 16 + r] = ss[mb];
-    }
-    __syncthreads();
   }
-  constexpr int UNITS = (EPI == EPI_SWIGLU ? 1 : NT) * MB * 64;
+  if (WK > 1 || NORM) __syncthreads();
+  constexpr int UNITS = (PAIRED ? 1 : NT) * MB * 64;
   for (int u = tid; u < UNITS; u += blockDim.x) {
     const int l = u & 63, mb = (u >> 6) % MB, t = (u >> 6) / MB;
     const int token = mb * 16 + (l & 15), qq = l >> 4;
     f32x4_t s0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, s1 = s0;
-    float total = 0.f;
     if (WK > 1) {
       for (int w = 0; w < WK; ++w) {
         s0 += red[(w * NT * MB + t * MB + mb) * 64 + l];
-        if (EPI == EPI_SWIGLU) s1 += red[(w * NT * MB + MB + mb) * 64 + l];
-        if (NORM) total += sq[w * 16 * MB + mb * 16 + (l & 15)];
+        if (PAIRED) s1 += red[(w * NT * MB + MB + mb) * 64 + l];
       }
     } else {
       // one wavefront: unit u is this very lane's accumulator (u < 64 * NT * MB, tid == lane)
@@ -259,25 +340,38 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
 #pragma unroll
         for (int mm = 0; mm < MB; ++mm) {
           if (tt == t && mm == mb) s0 = acc[tt][mm];
-          if (EPI == EPI_SWIGLU && tt == 1 && mm == mb) s1 = acc[tt][mm];
-          if (NORM && mm == mb) total = ss[mm];
+          if (PAIRED && tt == 1 && mm == mb) s1 = acc[tt][mm];
         }
     }
-    if (qq * 4 >= TH) continue;
-    const float scale = NORM ? 1.0f / sqrtf(total / (float)a.K + a.eps) : 1.0f;
-    const int n = (EPI == EPI_SWIGLU ? g : g * NT + t) * TH + qq * 4;
-    store4<EPI>(a, s0, s1, scale, token, n);
+    const float scale = NORM ? scales[token] : 1.0f;
+    const bool live = qq * 4 < TH && token < a.M;
+    if (EPI == EPI_ROPE) {
+      if (live) rope_store(a, s0 * scale, s1 * scale, token, rope_head, rope_col + qq * 4);
+    } else {
+      const int tile = PAIRED ? g : g * NT + t;
+      const int n = tile * TH + qq * 4;
+      if (EPI == EPI_RESIDUAL && a.emit_w != nullptr) {
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          x[j] = (live && n + j < a.N)
+                     ? round_to<bf16_t>(s0[j] * scale) + __bfloat162float(a.residual[(size_t)token * a.ldr + n + j])
+                     : 0.f;
+        emit_for_norm(a, x, live && n < a.N, token, n, tile, l);
+      }
+      if (live) store4<EPI>(a, s0, s1, scale, token, n);
+    }
   }
 }
 
 // ---------------------------------------------------------------------------------
-// 16 < M <= 128: A passes through LDS.
+// 16 < M <= 128 (and any M for a wide output): A passes through LDS.
 // A workgroup is 4 x WK wavefronts; wavefront (wn, wk) owns the NT tiles of index
 // (4 * workgroup + wn) * NT + t and the steps of K that row wk of the workgroup has.
 // A round is 4 steps; wavefront wn of a row brings step wn of the round into LDS in
 // the lane order of the matrix-core operand (one KB a unit), for all MB blocks of 16
 // tokens, while the round before is multiplied.
-// LDS: [squares: waves * 16 * MB floats][2 buffers x WK x 4 steps x MB units of 1 KB],
+// LDS: [scales: 16 * MB floats when NORM][2 buffers x WK x 4 steps x MB units of 1 KB],
 // the sums of the wavefront rows reuse the buffers after the last round.
 // ---------------------------------------------------------------------------------
 #define ST_WN 4
@@ -294,10 +388,11 @@ __global__ __launch_bounds__(1024) void gemm_staged_kernel(GemmArgs a) {
   const int K32 = (a.K + 31) >> 5;
   const int ks0 = (int)((long)K32 * wk / WK), ks1 = (int)((long)K32 * (wk + 1) / WK);
   const int rounds = ((K32 + WK - 1) / WK + ST_SC - 1) / ST_SC;
-  float* sq = (float*)smem;  // [wave][16 * MB]
-  unsigned char* stage = smem + (NORM ? (size_t)nwaves * 16 * MB * sizeof(float) : 0);
+  float* scales = (float*)smem;
+  unsigned char* stage = smem + (NORM ? 16 * MB * sizeof(float) : 0);
   bf16x8_t* stage_v = (bf16x8_t*)stage;  // [buffer][wk][step][mb][lane]
   f32x4_t* red = (f32x4_t*)stage;         // [wk][wn][NT * MB][lane], after the last round
+  if (NORM) row_scales<MB>(a, scales);
 
   const int unit = blockIdx.x * ST_WN + wn;  // SwiGLU: a pair of tiles; else NT tiles
   const bf16_t* wp[NT];
@@ -315,20 +410,14 @@ __global__ __launch_bounds__(1024) void gemm_staged_kernel(GemmArgs a) {
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) ap[mb] = a.A + (size_t)min(mb * 16 + r, a.M - 1) * a.lda + q * 8;
 
-  float ss[MB];  // squares of the values of row 16 mb + r that this lane has brought in
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) ss[mb] = 0.f;
-
   // this wavefront's step of a round of A, for every block of tokens
   auto load_a = [&](int round, bf16x8_t (&piece)[MB]) {
     const int s = ks0 + round * ST_SC + wn;
-    const int k = s * 32 + q * 8;
-    const bool ok = s < ks1 && k < a.K;
+    const bool ok = s < ks1 && s * 32 + q * 8 < a.K;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       if (ok) {
         piece[mb] = *(const bf16x8_t*)(ap[mb] + (size_t)s * 32);
-        if (NORM) piece[mb] = weigh_piece(piece[mb], a.norm_w, a.norm_w_f32, k, ss[mb]);
       } else {
         piece[mb] = zero8();
       }
@@ -396,33 +485,14 @@ __global__ __launch_bounds__(1024) void gemm_staged_kernel(GemmArgs a) {
     buf ^= 1;
   }
 
-  // every piece of A was brought in by one wavefront: the squares of a row are the sum over all
-  if (NORM) {
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      ss[mb] += __shfl_xor(ss[mb], 16, 64);
-      ss[mb] += __shfl_xor(ss[mb], 32, 64);
-      if (q == 0) sq[wave * 16 * MB + mb * 16 + r] = ss[mb];
-    }
-  }
   // add the rows' partial sums in row order
-  if (WK > 1) {
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) red[((size_t)(wk * ST_WN + wn) * NT * MB + t * MB + mb) * 64 + lane] = acc[t][mb];
-  }
-  if (WK > 1 || NORM) __syncthreads();
   constexpr int TN = (EPI == EPI_SWIGLU ? 1 : NT);
   if (WK == 1) {
     // every wavefront stores its own sums
     const int token0 = lane & 15, qq = lane >> 4;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      float total = 0.f;
-      if (NORM)
-        for (int w = 0; w < nwaves; ++w) total += sq[w * 16 * MB + mb * 16 + token0];
-      const float scale = NORM ? 1.0f / sqrtf(total / (float)a.K + a.eps) : 1.0f;
+      const float scale = NORM ? scales[mb * 16 + token0] : 1.0f;
 #pragma unroll
       for (int t = 0; t < TN; ++t) {
         const int n = (EPI == EPI_SWIGLU ? unit : unit * NT + t) * 16 + qq * 4;
@@ -431,6 +501,11 @@ __global__ __launch_bounds__(1024) void gemm_staged_kernel(GemmArgs a) {
     }
     return;
   }
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) red[((size_t)(wk * ST_WN + wn) * NT * MB + t * MB + mb) * 64 + lane] = acc[t][mb];
+  __syncthreads();
   constexpr int UNITS = ST_WN * TN * MB * 64;
   for (int u = tid; u < UNITS; u += blockDim.x) {
     const int l = u & 63;
@@ -444,10 +519,7 @@ __global__ __launch_bounds__(1024) void gemm_staged_kernel(GemmArgs a) {
       s0 += red[((size_t)(w * ST_WN + own) * NT * MB + t * MB + mb) * 64 + l];
       if (EPI == EPI_SWIGLU) s1 += red[((size_t)(w * ST_WN + own) * NT * MB + MB + mb) * 64 + l];
     }
-    float total = 0.f;
-    if (NORM)
-      for (int w = 0; w < nwaves; ++w) total += sq[w * 16 * MB + mb * 16 + (l & 15)];
-    const float scale = NORM ? 1.0f / sqrtf(total / (float)a.K + a.eps) : 1.0f;
+    const float scale = NORM ? scales[token] : 1.0f;
     const int tile_group = blockIdx.x * ST_WN + own;
     const int n = (EPI == EPI_SWIGLU ? tile_group : tile_group * NT + t) * 16 + qq * 4;
     store4<EPI>(a, s0, s1, scale, token, n);
@@ -466,7 +538,7 @@ static bool allow_lds(Kernel kernel, size_t lds) {
 template <int MB, int NT, int EPI, bool NORM>
 static bool launch_skinny_one(const GemmArgs& a, int groups, int WK, hipStream_t stream) {
   size_t lds = WK > 1 ? (size_t)WK * NT * MB * 64 * sizeof(f32x4_t) : 0;
-  if (NORM && WK > 1) lds += (size_t)WK * 16 * MB * sizeof(float);
+  if (NORM) lds += (size_t)16 * MB * sizeof(float);
   auto kernel = gemm_skinny_kernel<MB, NT, EPI, NORM>;
   if (!allow_lds(kernel, lds)) return false;
   hipLaunchKernelGGL(kernel, dim3(groups), dim3(WK * 64), lds, stream, a);
@@ -478,87 +550,130 @@ static bool launch_staged_one(const GemmArgs& a, int groups, int WK, hipStream_t
   size_t lds = (size_t)2 * WK * ST_SC * MB * 1024;
   const size_t red = WK > 1 ? (size_t)WK * ST_WN * NT * MB * 64 * sizeof(f32x4_t) : 0;
   if (red > lds) lds = red;
-  if (NORM) lds += (size_t)WK * ST_WN * 16 * MB * sizeof(float);
+  if (NORM) lds += (size_t)16 * MB * sizeof(float);
   auto kernel = gemm_staged_kernel<MB, NT, EPI, NORM>;
   if (!allow_lds(kernel, lds)) return false;
   hipLaunchKernelGGL(kernel, dim3(groups), dim3(WK * ST_WN * 64), lds, stream, a);
   return true;
 }
 
-template <int MB, int NT, bool STAGED>
-static bool launch_epi(const GemmArgs& a, int epi, bool norm, int groups, int WK, hipStream_t stream) {
-#define TK_GEMM_CASE(E)                                                                         \
-  if (STAGED)                                                                                   \
-    return norm ? launch_staged_one<MB, NT, E, true>(a, groups, WK, stream)                     \
-                : launch_staged_one<MB, NT, E, false>(a, groups, WK, stream);                   \
-  else                                                                                          \
-    return norm ? launch_skinny_one<MB, NT, E, true>(a, groups, WK, stream)                     \
-                : launch_skinny_one<MB, NT, E, false>(a, groups, WK, stream);
-  switch (epi) {
-    case EPI_STORE: TK_GEMM_CASE(EPI_STORE)
-    case EPI_RESIDUAL:
-      if (STAGED) return launch_staged_one<MB, NT, EPI_RESIDUAL, false>(a, groups, WK, stream);
-      return launch_skinny_one<MB, NT, EPI_RESIDUAL, false>(a, groups, WK, stream);
-    case EPI_F32: TK_GEMM_CASE(EPI_F32)
-    default: return false;
-  }
-#undef TK_GEMM_CASE
-}
-
+// the combinations that exist: a residual never follows a norm (the norm's product feeds a
+// mixer or a feed-forward first), the staged kernel has neither rotation nor residual
 template <int MB, bool STAGED>
 static bool launch_mb(const GemmArgs& a, int epi, bool norm, int NT, int groups, int WK, hipStream_t stream) {
-  if (epi == EPI_SWIGLU) {
-    if (STAGED)
-      return norm ? launch_staged_one<MB, 2, EPI_SWIGLU, true>(a, groups, WK, stream)
-                  : launch_staged_one<MB, 2, EPI_SWIGLU, false>(a, groups, WK, stream);
-    return norm ? launch_skinny_one<MB, 2, EPI_SWIGLU, true>(a, groups, WK, stream)
-                : launch_skinny_one<MB, 2, EPI_SWIGLU, false>(a, groups, WK, stream);
+#define TK_ONE(NTV, E, NV) \
+  (STAGED ? launch_staged_one<MB, NTV, (E == EPI_ROPE || E == EPI_RESIDUAL) ? EPI_STORE : E, NV>(a, groups, WK, stream) \
+          : launch_skinny_one<MB, NTV, E, NV>(a, groups, WK, stream))
+  switch (epi) {
+    case EPI_SWIGLU: return norm ? TK_ONE(2, EPI_SWIGLU, true) : TK_ONE(2, EPI_SWIGLU, false);
+    case EPI_ROPE: return STAGED ? false : (norm ? TK_ONE(2, EPI_ROPE, true) : TK_ONE(2, EPI_ROPE, false));
+    case EPI_RESIDUAL: return (STAGED || norm) ? false : (NT == 1 ? TK_ONE(1, EPI_RESIDUAL, false) : TK_ONE(2, EPI_RESIDUAL, false));
+    case EPI_STORE:
+      if (NT == 1) return norm ? TK_ONE(1, EPI_STORE, true) : TK_ONE(1, EPI_STORE, false);
+      return norm ? TK_ONE(2, EPI_STORE, true) : TK_ONE(2, EPI_STORE, false);
+    case EPI_F32:
+      if (NT == 1) return norm ? TK_ONE(1, EPI_F32, true) : TK_ONE(1, EPI_F32, false);
+      return norm ? TK_ONE(2, EPI_F32, true) : TK_ONE(2, EPI_F32, false);
+    default: return false;
   }
-  return NT == 1 ? launch_epi<MB, 1, STAGED>(a, epi, norm, groups, WK, stream)
-                 : launch_epi<MB, 2, STAGED>(a, epi, norm, groups, WK, stream);
+#undef TK_ONE
+}
+
+struct GemmExtra {
+  // norm in front
+  const float* sumsq_in;
+  int parts_in;
+  float eps;
+  // residual epilogue: for the norm that follows
+  const void* emit_w;
+  int emit_w_f32;
+  void* emit_scaled;
+  int ld_emit;
+  float* emit_sumsq;
+  int parts_out;
+  // rotation with append
+  const int* positions;
+  const int* token_req;
+  const int* block_table;
+  int table_stride;
+  const float* cos_t;
+  const float* sin_t;
+  void* kcache;
+  void* vcache;
+  int nq, nkv, d, P;
+};
+
+// Number of partial sums a row gets from the residual epilogue with emit_w: one a tile.
+TK_API int tk_gemm_skinny_parts(int M, int N, int tile_rows) {
+  const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
+  const int th = tile_rows > 0 ? tile_rows : ((MB == 1 && (N + 15) / 16 < 256) ? 8 : 16);
+  return (N + th - 1) / th;
 }
 
 // A [M, K] bfloat16 (rows lda apart), W [N, K] row-major ([2N, K] gate over up for SwiGLU),
-// C [M, N].  norm_w (may be null): RMSNorm weight [K] applied to A first, bfloat16 or
-// float (norm_w_f32).  waves_k: wavefronts (skinny) or wavefront rows (staged) that split
-// K inside a workgroup (0 = choose); tiles: weight tiles of 16 rows per wavefront, 1 or 2
-// (0 = choose; SwiGLU always pairs gate and up); staged: -1 = choose, 0 = skinny, 1 = staged;
-// tile_rows: weight rows of a tile that the skinny kernel uses, 16 or 8 (0 = choose).
+// C [M, N] ([M, nq * d] with the rotation epilogue).  `extra` (may be null) carries the
+// norm in front, the outputs for a following norm and the rotation's operands.
+// waves_k: wavefronts (skinny) or wavefront rows (staged) that split K inside a workgroup
+// (0 = choose); tiles: weight tiles per wavefront, 1 or 2 (0 = choose; SwiGLU and the rotation
+// always pair); staged: -1 = choose, 0 = skinny, 1 = staged; tile_rows: weight rows of a
+// tile that the skinny kernel uses, 16 or 8 (0 = choose; tk_gemm_skinny_parts tells the
+// choice to whoever sizes emit_sumsq).
 TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, int ldc,
-                                   const void* residual, int ldr, const void* norm_w,
-                                   int norm_w_f32, float eps, int M, int N, int K, int epi,
-                                   int waves_k, int tiles, int staged, int tile_rows,
-                                   hipStream_t stream) {
+                               const void* residual, int ldr, const GemmExtra* extra, int M, int N,
+                               int K, int epi, int waves_k, int tiles, int staged, int tile_rows,
+                               hipStream_t stream) {
   TK_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
   TK_REQUIRE(M <= 128, "gemm_skinny: at most 128 rows, got %d", M);
-  TK_REQUIRE(epi >= EPI_STORE && epi <= EPI_F32, "gemm_skinny: unknown epilogue %d", epi);
+  TK_REQUIRE(epi >= EPI_STORE && epi <= EPI_ROPE, "gemm_skinny: unknown epilogue %d", epi);
   TK_REQUIRE(K % 8 == 0, "gemm_skinny: K=%d must be a multiple of 8 for the bfloat16 kernels", K);
   TK_REQUIRE(lda % 8 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0,
              "gemm_skinny: rows of A and W must be 16-byte aligned (lda=%d)", lda);
-  TK_REQUIRE(!norm_w || ((uintptr_t)norm_w & 15) == 0, "gemm_skinny: the norm weight must be 16-byte aligned");
-  TK_REQUIRE(lda >= K && ldc >= N, "gemm_skinny: strides shorter than rows");
+  TK_REQUIRE(lda >= K, "gemm_skinny: lda %d shorter than K %d", lda, K);
   TK_REQUIRE(epi != EPI_RESIDUAL || (residual && ldr >= N), "gemm_skinny: residual missing or too narrow");
-  if (M == 0) return 0;
-  GemmArgs a;
-  a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.C = C; a.ldc = ldc;
-  a.residual = (const bf16_t*)residual; a.ldr = ldr; a.norm_w = norm_w; a.norm_w_f32 = norm_w_f32;
-  a.eps = eps; a.M = M; a.N = N; a.K = K; a.TH = 16;
   TK_REQUIRE(tile_rows == 0 || tile_rows == 8 || tile_rows == 16, "gemm_skinny: tile_rows %d is not 0, 8 or 16", tile_rows);
-  const bool norm = norm_w != nullptr;
+  if (M == 0) return 0;
+  GemmArgs a = {};
+  a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.C = C; a.ldc = ldc;
+  a.residual = (const bf16_t*)residual; a.ldr = ldr; a.M = M; a.N = N; a.K = K; a.TH = 16;
+  bool norm = false;
+  if (extra) {
+    a.sumsq_in = extra->sumsq_in; a.parts_in = extra->parts_in; a.eps = extra->eps;
+    a.emit_w = extra->emit_w; a.emit_w_f32 = extra->emit_w_f32; a.emit_scaled = (bf16_t*)extra->emit_scaled;
+    a.ld_emit = extra->ld_emit; a.emit_sumsq = extra->emit_sumsq; a.parts_out = extra->parts_out;
+    a.positions = extra->positions; a.token_req = extra->token_req; a.block_table = extra->block_table;
+    a.table_stride = extra->table_stride; a.cos_t = extra->cos_t; a.sin_t = extra->sin_t;
+    a.kcache = (bf16_t*)extra->kcache; a.vcache = (bf16_t*)extra->vcache;
+    a.nq = extra->nq; a.nkv = extra->nkv; a.d = extra->d; a.P = extra->P;
+    norm = a.sumsq_in != nullptr;
+  }
+  TK_REQUIRE(!norm || a.parts_in > 0, "gemm_skinny: a norm in front needs its partial sums");
+  TK_REQUIRE(!(norm && epi == EPI_RESIDUAL), "gemm_skinny: a norm in front cannot be combined with a residual behind");
+  TK_REQUIRE(a.emit_w == nullptr || (epi == EPI_RESIDUAL && a.emit_scaled && a.emit_sumsq && a.ld_emit >= N),
+             "gemm_skinny: outputs for a following norm go with the residual epilogue and need their buffers");
+  if (epi == EPI_ROPE) {
+    TK_REQUIRE(extra && a.positions && a.token_req && a.block_table && a.kcache && a.vcache,
+               "gemm_skinny: the rotation epilogue needs positions, the block table and the cache");
+    TK_REQUIRE(a.nq > 0 && a.nkv > 0 && a.d > 0 && a.d % 8 == 0 && a.P > 0 && N == (a.nq + 2 * a.nkv) * a.d,
+               "gemm_skinny: rotation epilogue with nq=%d nkv=%d d=%d does not match N=%d", a.nq, a.nkv, a.d, N);
+    TK_REQUIRE((a.cos_t == nullptr) == (a.sin_t == nullptr), "gemm_skinny: cos and sin tables go together");
+    TK_REQUIRE(ldc >= a.nq * a.d, "gemm_skinny: ldc %d shorter than the query heads", ldc);
+  } else {
+    TK_REQUIRE(ldc >= N, "gemm_skinny: ldc %d shorter than N %d", ldc, N);
+  }
 
   const int n16 = (N + 15) / 16;
   const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
   const int K32 = (K + 31) / 32;
-  const int n16_units = epi == EPI_SWIGLU ? n16 : n16;
   // measured on an MI355X: passing A through LDS pays for a wide output (the head) from 5 rows on,
   // where many wavefronts of a workgroup share it; a narrow one needs every tile in a workgroup of its own
-  const bool use_staged = (staged < 0 ? M > 4 && K32 >= 2 * ST_SC && n16_units >= 2048 : staged != 0);
-  TK_REQUIRE(!(norm && epi == EPI_RESIDUAL), "gemm_skinny: a norm in front cannot be combined with a residual behind");
-  int NT = epi == EPI_SWIGLU ? 2 : (tiles > 0 ? tiles : 1);
+  const bool can_stage = epi != EPI_ROPE && epi != EPI_RESIDUAL;
+  const bool use_staged = can_stage && (staged < 0 ? M > 4 && K32 >= 2 * ST_SC && n16 >= 2048 : staged != 0);
+  const bool paired = epi == EPI_SWIGLU || epi == EPI_ROPE;
+  int NT = paired ? 2 : (tiles > 0 ? tiles : 1);
   TK_REQUIRE(NT == 1 || NT == 2, "gemm_skinny: tiles=%d outside 1..2", NT);
-  const int units = epi == EPI_SWIGLU ? n16 : (n16 + NT - 1) / NT;  // what one wavefront (row) owns
   bool ok;
   if (use_staged) {
+    const int units = paired ? n16 : (n16 + NT - 1) / NT;  // what one wavefront row owns
     const int groups = (units + ST_WN - 1) / ST_WN;
     int WK = waves_k;
     if (WK <= 0) {
@@ -578,8 +693,15 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
     }
   } else {
     // fewer tiles than compute units: tiles of 8 rows make twice the workgroups
-    a.TH = tile_rows > 0 ? tile_rows : ((MB == 1 && units < 256) ? 8 : 16);
-    const int groups = a.TH == 16 ? units : (epi == EPI_SWIGLU ? (N + 7) / 8 : ((N + 7) / 8 + NT - 1) / NT);
+    a.TH = tile_rows > 0 ? tile_rows : ((MB == 1 && n16 < 256) ? 8 : 16);
+    const int th_units = (N + a.TH - 1) / a.TH;
+    int groups;
+    if (epi == EPI_ROPE) {
+      groups = (a.nq + 2 * a.nkv) * ((a.d / 2 + a.TH - 1) / a.TH);
+    } else {
+      groups = paired ? th_units : (th_units + NT - 1) / NT;
+    }
+    TK_REQUIRE(a.emit_w == nullptr || a.parts_out == th_units, "gemm_skinny: %d partial sums a row, the caller sized for %d", th_units, a.parts_out);
     int WK = waves_k;
     if (WK <= 0) {
       // a wavefront issues the loads of U steps together: best when that is all it has to do,
@@ -599,7 +721,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
       default: ok = launch_mb<8, false>(a, epi, norm, NT, groups, WK, stream); break;
     }
   }
-  TK_REQUIRE(ok, "gemm_skinny: the kernel's local memory could not be reserved");
+  TK_REQUIRE(ok, "gemm_skinny: no kernel for this combination, or its local memory could not be reserved");
   TK_CHECK_LAUNCH("gemm_skinny");
   return 0;
 }

@@ -6,7 +6,9 @@ step can be recorded into a HIP graph.
 
 from __future__ import annotations
 
+import ctypes
 import math
+from dataclasses import dataclass
 
 import torch
 
@@ -477,8 +479,48 @@ def sample(
 # bfloat16 matrix products on the matrix cores
 # --------------------------------------------------------------------------
 
-EPI_STORE, EPI_RESIDUAL, EPI_SWIGLU, EPI_F32 = 0, 1, 2, 3
+EPI_STORE, EPI_RESIDUAL, EPI_SWIGLU, EPI_F32, EPI_ROPE = 0, 1, 2, 3, 4
 SKINNY_MAX_ROWS = 128
+
+
+class _GemmExtra(ctypes.Structure):
+    """The optional operands of tk_gemm_skinny_bf16 (struct GemmExtra of gemm_mfma.hip)."""
+
+    _fields_ = [
+        ("sumsq_in", ctypes.c_void_p), ("parts_in", ctypes.c_int), ("eps", ctypes.c_float),
+        ("emit_w", ctypes.c_void_p), ("emit_w_f32", ctypes.c_int), ("emit_scaled", ctypes.c_void_p),
+        ("ld_emit", ctypes.c_int), ("emit_sumsq", ctypes.c_void_p), ("parts_out", ctypes.c_int),
+        ("positions", ctypes.c_void_p), ("token_req", ctypes.c_void_p), ("block_table", ctypes.c_void_p),
+        ("table_stride", ctypes.c_int), ("cos_t", ctypes.c_void_p), ("sin_t", ctypes.c_void_p),
+        ("kcache", ctypes.c_void_p), ("vcache", ctypes.c_void_p),
+        ("nq", ctypes.c_int), ("nkv", ctypes.c_int), ("d", ctypes.c_int), ("P", ctypes.c_int),
+    ]
+
+
+@dataclass
+class Prenorm:
+    """What a residual product leaves for the RMSNorm that follows it: the new rows
+    times the norm's weight (rounded once) and, per row, partial sums of squares."""
+
+    scaled: torch.Tensor  # [M, N] bfloat16
+    sumsq: torch.Tensor  # [M, parts] float32
+
+
+@dataclass
+class RopeAppend:
+    """Operands of the rotation-with-append epilogue (see rope_append)."""
+
+    positions: torch.Tensor
+    token_req: torch.Tensor
+    block_table: torch.Tensor
+    cos: torch.Tensor | None
+    sin: torch.Tensor | None
+    kcache: torch.Tensor
+    vcache: torch.Tensor
+    nq: int
+    nkv: int
+    head_dim: int
+    page_size: int
 
 
 def gemm_skinny_bf16(
@@ -487,27 +529,67 @@ def gemm_skinny_bf16(
     residual: torch.Tensor | None = None,
     out_f32: bool = False,
     swiglu: bool = False,
-    norm_weight: torch.Tensor | None = None,
+    prenorm: Prenorm | None = None,
     norm_eps: float = 0.0,
+    emit_weight: torch.Tensor | None = None,
+    rope: RopeAppend | None = None,
     waves_k: int = 0,
     tiles: int = 0,
     staged: int = -1,
     tile_rows: int = 0,
-) -> torch.Tensor:
+):
     """a [M <= 128, K] times w [N, K] transposed on the matrix cores, with the
-    epilogue fused: + residual, 32-bit output, or (``swiglu``: w is [gate | up]
-    stacked, 2I rows) silu(gate) * up -> [M, I].  ``norm_weight``: ``a`` is
-    RMS-normed with this weight and ``norm_eps`` on the way in."""
-    _gpu(a, w, residual)
+    epilogue fused: + residual, 32-bit output, (``swiglu``: w is [gate | up]
+    stacked, 2I rows) silu(gate) * up -> [M, I], or (``rope``: w is [q | k | v]
+    stacked) rotation of q and k with the append of k and v to the pages -> q [M, nq*d].
+
+    ``prenorm``: the product of RMSNorm(x): ``a`` must be ``prenorm.scaled`` and the
+    rows are divided by their rms (``norm_eps``) in the epilogue.  ``emit_weight``
+    (with ``residual``): the weight of the norm that follows; returns
+    ``(out, Prenorm)`` for it."""
+    _gpu(a, w, residual, emit_weight)
     _need(a.dim() == 2 and a.stride(1) == 1 and a.dtype == torch.bfloat16, "gemm_skinny: A must be bfloat16 [M, K]")
     _need(w.dim() == 2 and w.is_contiguous() and w.dtype == torch.bfloat16, "gemm_skinny: W must be contiguous bfloat16 [N, K]")
     m, k = a.shape
     _need(w.shape[1] == k, f"gemm_skinny: A has K={k}, W has K={w.shape[1]}")
     n = w.shape[0]
+    n_out = n
+    extra = _GemmExtra()
+    use_extra = False
     if swiglu:
-        _need(residual is None and not out_f32 and n % 2 == 0, "gemm_skinny: SwiGLU takes a [2I, K] weight, no residual, bfloat16 output")
+        _need(residual is None and not out_f32 and rope is None and n % 2 == 0,
+              "gemm_skinny: SwiGLU takes a [2I, K] weight, no residual, bfloat16 output")
         n //= 2
+        n_out = n
         epi = EPI_SWIGLU
+    elif rope is not None:
+        _need(residual is None and not out_f32, "gemm_skinny: the rotation epilogue stands alone")
+        epi = EPI_ROPE
+        r = rope
+        _gpu(r.positions, r.token_req, r.block_table, r.cos, r.sin, r.kcache, r.vcache)
+        _need(n == (r.nq + 2 * r.nkv) * r.head_dim, "gemm_skinny: W is not [q | k | v] of these head counts")
+        for t, name in ((r.positions, "positions"), (r.token_req, "token_req"), (r.block_table, "block_table")):
+            _i32(t, name)
+        _need(r.positions.numel() == m and r.token_req.numel() == m and r.block_table.dim() == 2,
+              "gemm_skinny: positions/token_req need one entry a row, block_table [requests, width]")
+        pages = r.kcache.shape[0]
+        _need(tuple(r.kcache.shape) == (pages, r.nkv, r.page_size, r.head_dim) and r.kcache.is_contiguous()
+              and tuple(r.vcache.shape) == (pages, r.nkv, r.head_dim, r.page_size) and r.vcache.is_contiguous()
+              and r.kcache.dtype == torch.bfloat16 and r.vcache.dtype == torch.bfloat16,
+              "gemm_skinny: the pages must be contiguous bfloat16 [pages, nkv, P, d] and [pages, nkv, d, P]")
+        if r.cos is not None:
+            half = r.head_dim // 2
+            _need(r.sin is not None and r.cos.dtype == torch.float32 and r.sin.dtype == torch.float32
+                  and r.cos.shape == r.sin.shape and r.cos.shape[1] == half and r.cos.is_contiguous() and r.sin.is_contiguous(),
+                  "gemm_skinny: cos/sin tables must be contiguous float32 [positions, d/2]")
+        extra.positions, extra.token_req = r.positions.data_ptr(), r.token_req.data_ptr()
+        extra.block_table, extra.table_stride = r.block_table.data_ptr(), r.block_table.stride(0)
+        extra.cos_t = r.cos.data_ptr() if r.cos is not None else None
+        extra.sin_t = r.sin.data_ptr() if r.sin is not None else None
+        extra.kcache, extra.vcache = r.kcache.data_ptr(), r.vcache.data_ptr()
+        extra.nq, extra.nkv, extra.d, extra.P = r.nq, r.nkv, r.head_dim, r.page_size
+        use_extra = True
+        n_out = r.nq * r.head_dim
     elif residual is not None:
         _need(not out_f32, "gemm_skinny: a residual cannot be combined with 32-bit output")
         _need(residual.shape == (m, n) and residual.stride(1) == 1 and residual.dtype == torch.bfloat16,
@@ -515,24 +597,37 @@ def gemm_skinny_bf16(
         epi = EPI_RESIDUAL
     else:
         epi = EPI_F32 if out_f32 else EPI_STORE
-    if norm_weight is not None:
-        _gpu(norm_weight)
-        _need(norm_weight.shape == (k,) and norm_weight.is_contiguous()
-              and norm_weight.dtype in (torch.bfloat16, torch.float32),
-              "gemm_skinny: the norm weight must be contiguous [K], bfloat16 or float32")
+    if prenorm is not None:
+        _gpu(prenorm.scaled, prenorm.sumsq)
         _need(residual is None, "gemm_skinny: a norm in front cannot be combined with a residual behind")
-    out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=a.device)
+        _need(prenorm.scaled.data_ptr() == a.data_ptr() and prenorm.sumsq.dtype == torch.float32
+              and prenorm.sumsq.dim() == 2 and prenorm.sumsq.shape[0] == m and prenorm.sumsq.is_contiguous(),
+              "gemm_skinny: a norm in front takes the producer's scaled rows as A and its partial sums [M, parts]")
+        extra.sumsq_in, extra.parts_in, extra.eps = prenorm.sumsq.data_ptr(), prenorm.sumsq.shape[1], float(norm_eps)
+        use_extra = True
+    emitted = None
+    if emit_weight is not None:
+        _need(epi == EPI_RESIDUAL, "gemm_skinny: outputs for a following norm go with the residual epilogue")
+        _need(emit_weight.shape == (n,) and emit_weight.is_contiguous() and emit_weight.dtype in (torch.bfloat16, torch.float32),
+              "gemm_skinny: the following norm's weight must be contiguous [N], bfloat16 or float32")
+        parts = load("mfma").tk_gemm_skinny_parts(m, n, tile_rows)
+        emitted = Prenorm(torch.empty((m, n), dtype=torch.bfloat16, device=a.device),
+                          torch.empty((m, parts), dtype=torch.float32, device=a.device))
+        extra.emit_w, extra.emit_w_f32 = emit_weight.data_ptr(), 1 if emit_weight.dtype == torch.float32 else 0
+        extra.emit_scaled, extra.ld_emit = emitted.scaled.data_ptr(), n
+        extra.emit_sumsq, extra.parts_out = emitted.sumsq.data_ptr(), parts
+        staged = 0  # only the skinny kernel has this epilogue
+        use_extra = True
+    out = torch.empty((m, n_out), dtype=torch.float32 if out_f32 else torch.bfloat16, device=a.device)
     call(
         "tk_gemm_skinny_bf16",
-        a.data_ptr(), a.stride(0), w.data_ptr(), out.data_ptr(), n,
+        a.data_ptr(), a.stride(0), w.data_ptr(), out.data_ptr(), n_out,
         residual.data_ptr() if residual is not None else None,
         residual.stride(0) if residual is not None else 0,
-        norm_weight.data_ptr() if norm_weight is not None else None,
-        1 if (norm_weight is not None and norm_weight.dtype == torch.float32) else 0,
-        float(norm_eps),
+        ctypes.byref(extra) if use_extra else None,
         m, n, k, epi, waves_k, tiles, staged, tile_rows, _stream(),
     )
-    return out
+    return (out, emitted) if emit_weight is not None else out
 
 
 def add(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:

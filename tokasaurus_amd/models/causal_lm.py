@@ -9,7 +9,7 @@ import torch
 from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.models.spec import ModelSpec
 from tokasaurus_amd.parts.base import BLOCKS, CacheNeed, CacheView, Part, StateNeed, StepContext, TensorSpec
-from tokasaurus_amd.parts.block import build_with_shared
+from tokasaurus_amd.parts.block import build_with_shared, stream_and_prepared
 from tokasaurus_amd.parts.embedding import LMHead, TokenEmbedding
 from tokasaurus_amd.parts.linear import Placer
 
@@ -63,10 +63,18 @@ class CausalLM:
     ) -> torch.Tensor:
         """Run the batch of ``ctx`` and return logits [len(want_rows), vocab] in 32-bit."""
         x = self.embedding.forward(ctx)
-        last = len(self.spec.run_order) - 1
-        for i, entry in enumerate(self.spec.run_order):
+        order = self.spec.run_order
+        last = len(order) - 1
+        prepared = None  # what a block has done for the norm that the next one (or the head) starts with
+        for i, entry in enumerate(order):
             rows = want_rows if i == last else None
-            x = self.blocks[entry.layer].forward(x, ctx, caches[i], states[i], rows)
+            block = self.blocks[entry.layer]
+            if block.fuses_norm:
+                next_norm = self.blocks[order[i + 1].layer].entry_norm() if i < last else self.head.norm
+                out = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared, next_norm=next_norm)
+            else:
+                out = block.forward(x, ctx, caches[i], states[i], rows)
+            x, prepared = stream_and_prepared(out)
         if last < 0:
             x = ops.gather_rows(x, want_rows)
-        return self.head.forward(x)
+        return self.head.forward(x, prepared)

@@ -10,6 +10,8 @@ from tokasaurus_amd.parts.base import (  # noqa: F401
     POSITION_ENCODINGS,
     CacheNeed,
     CacheView,
+    Normed,
+    Prepared,
     PartSpec,
     StateNeed,
     StepContext,

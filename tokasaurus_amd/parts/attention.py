@@ -22,6 +22,7 @@ from tokasaurus_amd.parts.base import (
     CacheNeed,
     CacheView,
     Mixer,
+    Normed,
     PartSpec,
     StepContext,
     TensorSpec,
@@ -60,6 +61,8 @@ def attention_plan(ctx: StepContext, group: int, nkv: int) -> AttentionPlan:
 
 @MIXERS.register("paged_attention")
 class PagedAttention(Mixer):
+    fuses_norm = True
+
     def __init__(
         self,
         hidden_size: int,
@@ -104,36 +107,44 @@ class PagedAttention(Mixer):
 
     def forward(
         self,
-        h: torch.Tensor,
+        h: torch.Tensor | Normed,
         residual: torch.Tensor,
         ctx: StepContext,
         cache: CacheView | None,
         state: torch.Tensor | None,
         rows: torch.Tensor | None,
-    ) -> torch.Tensor:
+        emit_norm=None,
+    ):
         assert cache is not None, "paged attention needs a cache"
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
-        # an entry that reads another entry's cache computes only its queries
-        qkv = self.qkv(h, rows=None if cache.writable else nq * d)
         cos = self.position.cos if self.position is not None else None
         sin = self.position.sin if self.position is not None else None
-        ops.rope_append(
-            qkv, ctx.positions, ctx.token_req, cache.block_table, cos, sin,
-            cache.keys, cache.values, nq, nkv, d, cache.page_size, write_cache=cache.writable,
-        )
-        if ops.attention_mfma_supports(qkv.dtype, d, cache.page_size):
+        q = None
+        if cache.writable:
+            # few rows in bfloat16: one kernel multiplies, rotates and appends
+            q = self.qkv.rope_append(h, ops.RopeAppend(
+                ctx.positions, ctx.token_req, cache.block_table, cos, sin, cache.keys, cache.values,
+                nq, nkv, d, cache.page_size))
+        if q is None:
+            # an entry that reads another entry's cache computes only its queries
+            q = self.qkv(h, rows=None if cache.writable else nq * d)
+            ops.rope_append(
+                q, ctx.positions, ctx.token_req, cache.block_table, cos, sin,
+                cache.keys, cache.values, nq, nkv, d, cache.page_size, write_cache=cache.writable,
+            )
+        if ops.attention_mfma_supports(q.dtype, d, cache.page_size):
             plan = attention_plan(ctx, nq // nkv, nkv)
             attn = ops.paged_attention_mfma(
-                qkv, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
+                q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
                 plan.tile_req, plan.tile_row0, plan.row_tiles, nq, nkv, d, cache.page_size,
                 plan.max_kv_len, plan.split, window=self.window, scale=self.scale, scratch=plan.scratch,
             )
         else:
             # the true 32-bit path, and shapes the matrix-core kernel does not take
             attn = ops.paged_attention_generic(
-                qkv, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
+                q, cache.keys, cache.values, cache.block_table, ctx.token_req, ctx.positions,
                 nq, nkv, d, cache.page_size, window=self.window, scale=self.scale,
             )
         if rows is not None:
             attn = ops.gather_rows(attn, rows)
-        return self.out(attn, residual=residual)
+        return self.out.with_residual(attn, residual, emit_norm)

@@ -109,6 +109,40 @@ class StepContext:
 
 
 # --------------------------------------------------------------------------
+# a norm that has not been applied yet
+# --------------------------------------------------------------------------
+
+
+@dataclass
+class Prepared:
+    """What the product in front of a norm has already done for it (the rows times the
+    norm's weight, and partial sums of their squares): ``data`` is the kernels' own
+    record (``kernels.ops.Prenorm``), ``norm`` the norm it was made for."""
+
+    data: Any
+    norm: "Norm"
+
+
+@dataclass
+class Normed:
+    """Rows that still have to pass ``norm``.  A part that says ``fuses_norm`` gets this
+    instead of normed rows and may fold the norm into its first product (a product
+    takes ``prepared`` when it is there and was made for this very norm); any part may
+    call ``materialize()`` and go on with plain rows."""
+
+    x: torch.Tensor
+    norm: "Norm"
+    prepared: Prepared | None = None
+
+    def usable(self) -> Prepared | None:
+        p = self.prepared
+        return p if p is not None and p.norm is self.norm and getattr(self.norm, "fusable_rms", False) else None
+
+    def materialize(self) -> torch.Tensor:
+        return self.norm.forward(self.x)
+
+
+# --------------------------------------------------------------------------
 # interfaces
 # --------------------------------------------------------------------------
 
@@ -150,7 +184,13 @@ class Mixer(Part):
     is given only those tokens' outputs are needed (the last block of a step
     keeps only the rows whose logits are wanted), but every token must still
     update the cache or state.
+
+    A mixer (or feed-forward) with ``fuses_norm = True`` takes ``h`` as a ``Normed``
+    and a keyword ``emit_norm`` (the norm that will be applied to its result, or
+    None) and may return ``(stream, Prepared)`` instead of the stream alone.
     """
+
+    fuses_norm = False
 
     def cache_need(self) -> CacheNeed | None:
         return None
@@ -171,16 +211,27 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """Token-wise transformation: returns ``residual + ff(h)``."""
+    """Token-wise transformation: returns ``residual + ff(h)`` (see ``Mixer`` for ``fuses_norm``)."""
+
+    fuses_norm = False
 
     def forward(self, h: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
 
 class Block(Part):
-    """The arrangement of norms, a mixer and a feed-forward around the residual stream."""
+    """The arrangement of norms, a mixer and a feed-forward around the residual stream.
+
+    A block with ``fuses_norm = True`` takes the keywords ``prepared`` (what the block
+    before has done for this block's first norm) and ``next_norm`` (the norm the model
+    applies to this block's result) and may return ``(stream, Prepared)``;
+    ``entry_norm()`` is the norm it applies to its input first."""
 
     mixer: Mixer
+    fuses_norm = False
+
+    def entry_norm(self) -> "Norm | None":
+        return None
 
     def forward(
         self,

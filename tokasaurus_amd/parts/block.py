@@ -20,7 +20,9 @@ from tokasaurus_amd.parts.base import (
     NORMS,
     Block,
     CacheView,
+    Normed,
     Part,
+    Prepared,
     PartSpec,
     StepContext,
     TensorSpec,
@@ -36,8 +38,15 @@ def build_with_shared(registry, spec: PartSpec, shared: dict):
     return registry.build(spec)
 
 
+def stream_and_prepared(out) -> tuple[torch.Tensor, Prepared | None]:
+    """A part returns the stream alone, or the stream with what it prepared for the next norm."""
+    return out if isinstance(out, tuple) else (out, None)
+
+
 @BLOCKS.register("pre_norm")
 class PreNormBlock(Block):
+    fuses_norm = True
+
     def __init__(
         self,
         mixer_norm: PartSpec,
@@ -62,6 +71,9 @@ class PreNormBlock(Block):
         for c in self.children():
             c.load(tensors, placer)
 
+    def entry_norm(self):
+        return self.mixer_norm
+
     def forward(
         self,
         x: torch.Tensor,
@@ -69,9 +81,16 @@ class PreNormBlock(Block):
         cache: CacheView | None,
         state: torch.Tensor | None,
         rows: torch.Tensor | None,
-    ) -> torch.Tensor:
-        h = self.mixer_norm.forward(x)
+        prepared: Prepared | None = None,
+        next_norm=None,
+    ):
         residual = x if rows is None else ops.gather_rows(x, rows)
-        x = self.mixer.forward(h, residual, ctx, cache, state, rows)
-        h = self.ff_norm.forward(x)
-        return self.feed_forward.forward(h, x)
+        if self.mixer.fuses_norm:
+            out = self.mixer.forward(Normed(x, self.mixer_norm, prepared), residual, ctx, cache, state, rows,
+                                     emit_norm=self.ff_norm)
+        else:
+            out = self.mixer.forward(self.mixer_norm.forward(x), residual, ctx, cache, state, rows)
+        x, prepared = stream_and_prepared(out)
+        if self.feed_forward.fuses_norm:
+            return self.feed_forward.forward(Normed(x, self.ff_norm, prepared), x, emit_norm=next_norm)
+        return self.feed_forward.forward(self.ff_norm.forward(x), x)

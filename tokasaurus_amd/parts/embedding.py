@@ -11,7 +11,7 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.kernels import ops
-from tokasaurus_amd.parts.base import MATRIX, NORMS, Part, PartSpec, StepContext, TensorSpec
+from tokasaurus_amd.parts.base import MATRIX, NORMS, Normed, Part, PartSpec, Prepared, StepContext, TensorSpec
 from tokasaurus_amd.parts.linear import Linear, Placer
 
 
@@ -52,5 +52,5 @@ class LMHead(Part):
         self.norm.load(tensors, placer)
         self.proj.load(tensors, placer)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.proj(self.norm.forward(x), out_f32=True)
+    def forward(self, x: torch.Tensor, prepared: Prepared | None = None) -> torch.Tensor:
+        return self.proj(Normed(x, self.norm, prepared), out_f32=True)

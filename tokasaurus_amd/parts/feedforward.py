@@ -5,12 +5,14 @@ from __future__ import annotations
 
 import torch
 
-from tokasaurus_amd.parts.base import FEED_FORWARDS, FeedForward, TensorSpec
+from tokasaurus_amd.parts.base import FEED_FORWARDS, FeedForward, Normed, TensorSpec
 from tokasaurus_amd.parts.linear import Linear, Placer
 
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    fuses_norm = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, names: dict[str, str]):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
@@ -24,5 +26,5 @@ class SwiGLU(FeedForward):
         self.gate_up.load(tensors, placer)
         self.down.load(tensors, placer)
 
-    def forward(self, h: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
-        return self.down(self.gate_up(h, swiglu=True), residual=residual)
+    def forward(self, h: torch.Tensor | Normed, residual: torch.Tensor, emit_norm=None):
+        return self.down.with_residual(self.gate_up(h, swiglu=True), residual, emit_norm)

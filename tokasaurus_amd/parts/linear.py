@@ -6,7 +6,9 @@ be stacked along the output rows into one product (q|k|v, gate|up).
 Which kernel runs is decided by the storage type and the number of rows:
   * float32: 32-bit multiply-adds throughout (the true 32-bit path);
   * bfloat16, up to 128 rows (decode): the hand-written matrix-core kernel that
-    streams the weight once and fuses the epilogue;
+    streams the weight once and fuses the epilogue; it can also fold in the norm in
+    front (``Normed`` input), leave what the norm behind it needs (``emit_norm``), and
+    rotate and append q, k and v (``rope_append``);
   * bfloat16, more rows (prefill): the library's matrix product, as in the
     reference (its projections are library calls), followed by the epilogue kernel.
 """
@@ -16,7 +18,7 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.kernels import ops
-from tokasaurus_amd.parts.base import MATRIX, TensorSpec
+from tokasaurus_amd.parts.base import MATRIX, Norm, Normed, Prepared, TensorSpec
 
 
 class Placer:
@@ -63,9 +65,12 @@ class Linear:
 
         self.weight = placer.place(("row_major", *self.names), make)
 
+    def _fast(self, m: int) -> bool:
+        return self.weight.dtype == torch.bfloat16 and 0 < m <= ops.SKINNY_MAX_ROWS
+
     def __call__(
         self,
-        x: torch.Tensor,
+        x: torch.Tensor | Normed,
         residual: torch.Tensor | None = None,
         out_f32: bool = False,
         rows: int | None = None,
@@ -75,14 +80,23 @@ class Linear:
         product rounded to the storage type first).  ``out_f32``: 32-bit output.
         ``swiglu``: the weight is [gate | up]; returns silu(gate) * up.
         ``rows`` limits the product to the first output rows of the stacked
-        weight (a mixer that only needs its queries)."""
+        weight (a mixer that only needs its queries).  ``x`` may be a ``Normed``:
+        the norm is folded into the product when it was prepared, else applied first."""
         w = self.weight
         if rows is not None and rows != self.total_out:
             w = w[:rows]
+        prenorm, eps = None, 0.0
+        if isinstance(x, Normed):
+            prepared = x.usable() if (self._fast(x.x.shape[0]) and residual is None) else None
+            if prepared is not None:
+                prenorm, eps, x = prepared.data, x.norm.eps, prepared.data.scaled
+            else:
+                x = x.materialize()
         m = x.shape[0]
         if w.dtype == torch.bfloat16 and m > 0:
             if m <= ops.SKINNY_MAX_ROWS:
-                return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu)
+                return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu,
+                                            prenorm=prenorm, norm_eps=eps)
             prod = torch.mm(x, w.t())  # library matrix product (hipBLASLt), 32-bit accumulation
             if swiglu:
                 return ops.swiglu(prod)
@@ -91,3 +105,29 @@ class Linear:
             return prod.float() if out_f32 else prod
         out = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)
         return ops.swiglu(out) if swiglu else out
+
+    def with_residual(
+        self, x: torch.Tensor, residual: torch.Tensor, emit_norm: Norm | None
+    ) -> tuple[torch.Tensor, Prepared | None]:
+        """residual + product and, where the kernel can, what ``emit_norm`` (the norm
+        that will be applied to the result) needs so that it costs no kernel of its own."""
+        if emit_norm is not None and getattr(emit_norm, "fusable_rms", False) and self._fast(x.shape[0]):
+            out, data = ops.gemm_skinny_bf16(x, self.weight, residual=residual, emit_weight=emit_norm.weight)
+            return out, Prepared(data, emit_norm)
+        return self(x, residual=residual), None
+
+    def rope_append(self, x: torch.Tensor | Normed, rope: "ops.RopeAppend") -> torch.Tensor | None:
+        """For a stacked [q | k | v] weight: the product with the rotation of q and k and the
+        append of k and v to the pages in its epilogue; returns q [M, nq*d], or None when
+        that kernel does not take this case (the caller then does the steps one by one)."""
+        m = (x.x if isinstance(x, Normed) else x).shape[0]
+        if not self._fast(m) or rope.head_dim % 2:
+            return None
+        prenorm, eps = None, 0.0
+        if isinstance(x, Normed):
+            prepared = x.usable()
+            if prepared is not None:
+                prenorm, eps, x = prepared.data, x.norm.eps, prepared.data.scaled
+            else:
+                x = x.materialize()
+        return ops.gemm_skinny_bf16(x, self.weight, rope=rope, prenorm=prenorm, norm_eps=eps)

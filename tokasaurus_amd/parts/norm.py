@@ -12,6 +12,8 @@ from tokasaurus_amd.parts.linear import Placer
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    fusable_rms = True  # weight and eps are all a product needs to fold this norm in
+
     def __init__(self, size: int, eps: float, name: str):
         self.size = size
         self.eps = float(eps)
