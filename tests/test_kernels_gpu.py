@@ -33,7 +33,7 @@ ATTN_CASES = [
 ]
 
 
-def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1):
+def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1, waves=1):
     from tokasaurus_amd.kernels import ops
 
     dtype = torch.bfloat16 if kind != "generic_f32" else torch.float32
@@ -46,24 +46,26 @@ def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=N
         return ops.paged_attention_generic(q, kc, vc, table, token_req, positions, nq, nkv, d, page, window=window)
     tile_req, tile_row0 = ops.attention_tiles(q_lens, nq // nkv, row_tiles)
     max_kv = max(kv_lens)
-    split = split or ops.attention_split(max_kv, len(tile_req), nkv)
+    if split is None:
+        split, waves = ops.attention_split(max_kv, len(tile_req), nkv)
     return ops.paged_attention_mfma(
         q, kc, vc, table, dev(case["q_start"]), dev(case["kv_len"]),
         torch.tensor(tile_req, dtype=torch.int32).cuda(), torch.tensor(tile_row0, dtype=torch.int32).cuda(),
-        row_tiles, nq, nkv, d, page, max_kv, split, window=window,
+        row_tiles, nq, nkv, d, page, max_kv, split, window=window, waves=waves,
     )
 
 
 @pytest.mark.parametrize("case_id", range(len(ATTN_CASES)))
-@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma", "mfma_split32", "mfma_rt2"])
+@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma", "mfma_split32", "mfma_rt2", "mfma_waves4", "mfma_waves16"])
 def test_paged_attention(kind, case_id):
     q_lens, kv_lens, nq, nkv, d, page, window = ATTN_CASES[case_id]
     dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
     case = make_paged_case(q_lens, kv_lens, nq, nkv, d, page, seed=case_id, dtype=dtype)
     ref = attention_reference(case, q_lens, kv_lens, nq, nkv, d, window=window)
-    split = 32 if kind == "mfma_split32" else (64 if kind == "mfma_rt2" else None)
+    split = {"mfma_split32": 32, "mfma_rt2": 64, "mfma_waves4": 256, "mfma_waves16": 512}.get(kind)
+    waves = {"mfma_waves4": 4, "mfma_waves16": 16}.get(kind, 1)
     got = run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=split,
-                        row_tiles=2 if kind == "mfma_rt2" else 1).float().cpu()
+                        row_tiles=2 if kind == "mfma_rt2" else 1, waves=waves).float().cpu()
     assert torch.isfinite(got).all()
     # values are of order 1; bfloat16 rounds the probabilities and the output to 8 bits
     tol = dict(atol=2e-5, rtol=1e-4) if kind == "generic_f32" else dict(atol=2e-2, rtol=2e-2)

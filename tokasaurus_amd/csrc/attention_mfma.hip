@@ -17,9 +17,12 @@
 //   K pages: [page][kv head][P][d]      V pages: [page][kv head][d][P], P % 4 == 0
 //
 // Splits.  The keys of a tile are cut at absolute multiples of `split`; each
-// (tile, kv head, split) is one wavefront.  A tile with one split writes the
-// output; otherwise partial (max, sum, weighted values) go to scratch and a
-// second kernel adds them in split order.
+// (tile, kv head, split) is one workgroup of NW wavefronts, which cut the split's
+// keys into NW consecutive parts (multiples of 32) and add their results through
+// LDS in wavefront order.  A tile with one split writes the output; otherwise
+// partial (max, sum, weighted values) go to scratch and a second kernel adds them
+// in split order.  With few tiles (decode) many wavefronts with two or three steps
+// each keep enough loads in flight; with many tiles (prompts) NW is 1.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -112,18 +115,22 @@ __device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, co
 }
 
 template <int DT, int RT>
-__global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
+__global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) {
+  extern __shared__ __align__(16) float wg_part[];  // [wavefront][16 * RT rows][D + 4], when NW > 1
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head size
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int NW = blockDim.x >> 6;
   const int r = lane & 15, q = lane >> 4;
   const int tile = blockIdx.x, kvh = blockIdx.y;
   const TileRange t = tile_range(a, tile, 16 * RT);
   const int s = t.s_first + blockIdx.z;
   if (s > t.s_last) return;
   const int nsp = t.s_last - t.s_first + 1;
-  const int k_begin = max((t.lo >> 5) << 5, s * a.split);
-  const int k_end = min(t.hi + 1, (s + 1) * a.split);
+  // this wavefront's part of the split: `sub` keys, a multiple of 32
+  const int sub = a.split / NW;
+  const int k_begin = max((t.lo >> 5) << 5, s * a.split + wave * sub);
+  const int k_end = min(t.hi + 1, s * a.split + (wave + 1) * sub);
   const int* table = a.block_table + (size_t)t.req * a.table_stride;
   const int P = a.P;
 
@@ -245,6 +252,45 @@ __global__ __launch_bounds__(64) void paged_attention_mfma_kernel(AttnArgs a) {
     float l = l_run[rt];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
+    l_run[rt] = l;
+  }
+  if (NW > 1) {
+    // every wavefront leaves (max, sum, weighted values) of its rows; wavefront 0 adds them in order
+    constexpr int ROW = D + 4;  // max, sum, two unused, then the values (16-byte aligned)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float* row = wg_part + ((size_t)wave * 16 * RT + rt * 16 + r) * ROW;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(f32x4_t*)(row + 4 + dt * 16 + q * 4) = acc[rt][dt];
+      if (q == 0) {
+        row[0] = m_run[rt];
+        row[1] = l_run[rt];
+      }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float m = -INFINITY;
+      for (int w = 0; w < NW; ++w) m = fmaxf(m, wg_part[((size_t)w * 16 * RT + rt * 16 + r) * ROW]);
+      float l = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int w = 0; w < NW; ++w) {
+        const float* row = wg_part + ((size_t)w * 16 * RT + rt * 16 + r) * ROW;
+        const float mw = row[0];
+        const float f = (mw == -INFINITY) ? 0.f : __expf(mw - m);
+        l += f * row[1];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[rt][dt] += f * *(const f32x4_t*)(row + 4 + dt * 16 + q * 4);
+      }
+      m_run[rt] = m;
+      l_run[rt] = l;
+    }
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const float l = l_run[rt];
     const int flat = t.row0 + rt * 16 + r;
     if (flat >= t.n_rows) continue;
     if (nsp == 1) {
@@ -314,27 +360,32 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D,
 }
 
 template <int DT, int RT>
-static void launch_attn(const AttnArgs& a, int grid_splits, hipStream_t stream) {
-  hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, RT>), dim3(a.n_tiles, a.nkv, grid_splits),
-                     dim3(64), 0, stream, a);
+static bool launch_attn(const AttnArgs& a, int grid_splits, int nw, hipStream_t stream) {
+  const size_t lds = nw > 1 ? (size_t)nw * 16 * RT * (DT * 16 + 4) * sizeof(float) : 0;
+  auto kernel = paged_attention_mfma_kernel<DT, RT>;
+  if (lds > 64 * 1024 &&
+      hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return false;
+  hipLaunchKernelGGL(kernel, dim3(a.n_tiles, a.nkv, grid_splits), dim3(64 * nw), lds, stream, a);
+  return true;
 }
 
 template <int RT>
-static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, hipStream_t stream) {
+static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, int nw, hipStream_t stream) {
   switch (dt) {
-    case 1: launch_attn<1, RT>(a, grid_splits, stream); return true;
-    case 2: launch_attn<2, RT>(a, grid_splits, stream); return true;
-    case 3: launch_attn<3, RT>(a, grid_splits, stream); return true;
-    case 4: launch_attn<4, RT>(a, grid_splits, stream); return true;
-    case 5: launch_attn<5, RT>(a, grid_splits, stream); return true;
-    case 6: launch_attn<6, RT>(a, grid_splits, stream); return true;
-    case 7: launch_attn<7, RT>(a, grid_splits, stream); return true;
-    case 8: launch_attn<8, RT>(a, grid_splits, stream); return true;
+    case 1: return launch_attn<1, RT>(a, grid_splits, nw, stream);
+    case 2: return launch_attn<2, RT>(a, grid_splits, nw, stream);
+    case 3: return launch_attn<3, RT>(a, grid_splits, nw, stream);
+    case 4: return launch_attn<4, RT>(a, grid_splits, nw, stream);
+    case 5: return launch_attn<5, RT>(a, grid_splits, nw, stream);
+    case 6: return launch_attn<6, RT>(a, grid_splits, nw, stream);
+    case 7: return launch_attn<7, RT>(a, grid_splits, nw, stream);
+    case 8: return launch_attn<8, RT>(a, grid_splits, nw, stream);
     default: return false;
   }
 }
 
-// Rows per tile are 16 * row_tiles (1 or 2).  `tile_req`/`tile_row0` list the
+// Rows per tile are 16 * row_tiles (1 or 2); `waves` wavefronts share a split.  `tile_req`/`tile_row0` list the
 // tiles; `grid_splits` is an upper bound on the splits of any tile and
 // `max_splits` the number the scratch has room for (grid_splits <= max_splits).
 // part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
@@ -346,13 +397,17 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
                                        const int* q_start, const int* kv_len,
                                        const int* tile_req, const int* tile_row0, int n_tiles,
                                        int row_tiles, int nq, int nkv, int d, int P, int window,
-                                       float scale, int split, int grid_splits, int max_splits,
+                                       float scale, int split, int waves, int grid_splits, int max_splits,
                                        float* part_o, float* part_ml, hipStream_t stream) {
   TK_REQUIRE(n_tiles >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_mfma: bad sizes tiles=%d nq=%d nkv=%d", n_tiles, nq, nkv);
   TK_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attention_mfma: head size %d is not a multiple of 16 up to 128", d);
   TK_REQUIRE(P > 0 && P % 4 == 0, "attention_mfma: page size %d is not a multiple of 4", P);
   TK_REQUIRE(row_tiles == 1 || row_tiles == 2, "attention_mfma: row_tiles %d outside 1..2", row_tiles);
   TK_REQUIRE(split > 0 && split % 32 == 0, "attention_mfma: split %d is not a multiple of 32", split);
+  TK_REQUIRE(waves >= 1 && waves <= 16 && split % (32 * waves) == 0,
+             "attention_mfma: %d wavefronts do not cut a split of %d keys into multiples of 32", waves, split);
+  TK_REQUIRE((size_t)waves * 16 * row_tiles * (d + 4) * sizeof(float) <= 160 * 1024 || waves == 1,
+             "attention_mfma: %d wavefronts of head size %d do not fit the local memory", waves, d);
   TK_REQUIRE(grid_splits >= 1 && grid_splits <= max_splits && grid_splits < 65536, "attention_mfma: splits %d of %d", grid_splits, max_splits);
   TK_REQUIRE(max_splits == 1 || (part_o && part_ml), "attention_mfma: split tiles need scratch");
   TK_REQUIRE(q_stride >= nq * d && out_stride >= nq * d && q_stride % 8 == 0 && out_stride % 4 == 0,
@@ -368,8 +423,8 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
   a.tile_req = tile_req; a.tile_row0 = tile_row0; a.n_tiles = n_tiles;
   a.nq = nq; a.nkv = nkv; a.group = nq / nkv; a.P = P; a.window = window; a.scale = scale;
   a.split = split; a.max_splits = max_splits; a.part_o = part_o; a.part_ml = part_ml;
-  const bool ok = row_tiles == 1 ? launch_attn_d<1>(a, d / 16, grid_splits, stream)
-                                 : launch_attn_d<2>(a, d / 16, grid_splits, stream);
+  const bool ok = row_tiles == 1 ? launch_attn_d<1>(a, d / 16, grid_splits, waves, stream)
+                                 : launch_attn_d<2>(a, d / 16, grid_splits, waves, stream);
   TK_REQUIRE(ok, "attention_mfma: no kernel for head size %d", d);
   TK_CHECK_LAUNCH("paged_attention_mfma");
   if (max_splits > 1) {

@@ -315,17 +315,19 @@ def attention_tiles(q_lens: list[int], group: int, row_tiles: int) -> tuple[list
     return tile_req, tile_row0
 
 
-def attention_split(max_kv_len: int, n_tiles: int, nkv: int) -> int:
-    """Keys per split (a multiple of 128).  With few tiles the keys are split so
-    that several thousand wavefronts share the work (measured best on an MI355X:
-    256 keys up to batch 8 at 8192 keys, 512 at batch 64); with thousands of
-    tiles (prompts) nothing is split."""
+def attention_split(max_kv_len: int, n_tiles: int, nkv: int) -> tuple[int, int]:
+    """(keys per split, wavefronts per workgroup).  With few tiles (decode) the keys are
+    cut so that about four thousand wavefronts share the work, each with 64 to 512
+    keys, 4 to 16 of them a workgroup (measured best on an MI355X at 8192 keys:
+    64 keys x 4 at batch 1, 128 x 8 at batch 8, 512 x 16 at batch 64); with thousands
+    of tiles (prompts) nothing is split and a workgroup is one wavefront."""
     base = max(n_tiles * nkv, 1)
     whole = -(-max(max_kv_len, 1) // 128) * 128
     if base >= 2048:
-        return whole
-    per = -(-(max_kv_len * base // 8192) // 128) * 128
-    return min(whole, max(256, per))
+        return whole, 1
+    sub = min(512, max(64, -(-(max_kv_len * base // 4096) // 32) * 32))
+    waves = 4 if base <= 16 else (8 if base <= 128 else 16)
+    return sub * waves, waves
 
 
 class AttentionScratch:
@@ -372,6 +374,7 @@ def paged_attention_mfma(
     split: int,
     window: int = 0,
     scale: float | None = None,
+    waves: int = 1,
     out: torch.Tensor | None = None,
     scratch: "AttentionScratch | None" = None,
 ) -> torch.Tensor:
@@ -404,6 +407,8 @@ def paged_attention_mfma(
     _need(attention_mfma_supports(q.dtype, head_dim, page_size),
           f"attention_mfma: head size {head_dim} / page size {page_size} not supported")
     _need(split > 0 and split % 32 == 0, "attention_mfma: split must be a positive multiple of 32")
+    _need(1 <= waves <= 16 and split % (32 * waves) == 0,
+          "attention_mfma: the wavefronts of a workgroup must cut a split into multiples of 32 keys")
     if out is None:
         out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
     else:
@@ -422,7 +427,7 @@ def paged_attention_mfma(
         q_start.data_ptr(), kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(),
         n_tiles, row_tiles, nq, nkv, head_dim, page_size, int(window),
         float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
-        split, max_splits, max_splits,
+        split, waves, max_splits, max_splits,
         part_o.data_ptr() if part_o is not None else None,
         part_ml.data_ptr() if part_ml is not None else None,
         _stream(),

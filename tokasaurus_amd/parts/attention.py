@@ -40,6 +40,7 @@ class AttentionPlan:
     row_tiles: int
     max_kv_len: int
     split: int
+    waves: int
     scratch: ops.AttentionScratch | None = None  # a replayed step keeps its own
 
 
@@ -51,8 +52,8 @@ def attention_plan(ctx: StepContext, group: int, nkv: int) -> AttentionPlan:
         row_tiles = 2 if ctx.max_q_len * group > 16 else 1
         tile_req, tile_row0 = ops.attention_tiles(q_lens, group, row_tiles)
         tiles = torch.tensor([tile_req, tile_row0], dtype=torch.int32).to(ctx.device)
-        split = ops.attention_split(ctx.max_kv_len, len(tile_req), nkv)
-        plan = AttentionPlan(tiles[0], tiles[1], row_tiles, ctx.max_kv_len, split)
+        split, waves = ops.attention_split(ctx.max_kv_len, len(tile_req), nkv)
+        plan = AttentionPlan(tiles[0], tiles[1], row_tiles, ctx.max_kv_len, split, waves)
         if ctx.extras.get("static"):
             plan.scratch = ops.AttentionScratch(ctx.device)
         ctx.extras[key] = plan
@@ -137,7 +138,7 @@ class PagedAttention(Mixer):
             attn = ops.paged_attention_mfma(
                 q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
                 plan.tile_req, plan.tile_row0, plan.row_tiles, nq, nkv, d, cache.page_size,
-                plan.max_kv_len, plan.split, window=self.window, scale=self.scale, scratch=plan.scratch,
+                plan.max_kv_len, plan.split, window=self.window, scale=self.scale, waves=plan.waves, scratch=plan.scratch,
             )
         else:
             # the true 32-bit path, and shapes the matrix-core kernel does not take
