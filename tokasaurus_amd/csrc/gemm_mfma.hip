@@ -630,7 +630,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
              "gemm_skinny: rows of A and W must be 16-byte aligned (lda=%d)", lda);
   TK_REQUIRE(lda >= K, "gemm_skinny: lda %d shorter than K %d", lda, K);
   TK_REQUIRE(epi != EPI_RESIDUAL || (residual && ldr >= N), "gemm_skinny: residual missing or too narrow");
-  TK_REQUIRE(tile_rows == 0 || tile_rows == 8 || tile_rows == 16, "gemm_skinny: tile_rows %d is not 0, 8 or 16", tile_rows);
+  TK_REQUIRE(tile_rows == 0 || tile_rows == 4 || tile_rows == 8 || tile_rows == 16, "gemm_skinny: tile_rows %d is not 0, 4, 8 or 16", tile_rows);
   if (M == 0) return 0;
   GemmArgs a = {};
   a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.C = C; a.ldc = ldc;

@@ -97,11 +97,12 @@ class Linear:
             if m <= ops.SKINNY_MAX_ROWS:
                 return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu,
                                             prenorm=prenorm, norm_eps=eps)
-            prod = torch.mm(x, w.t())  # library matrix product (hipBLASLt), 32-bit accumulation
+            # library matrix product (hipBLASLt), 32-bit accumulation
+            if residual is not None:
+                return torch.addmm(residual, x, w.t())  # the residual is added in the product's epilogue
+            prod = torch.mm(x, w.t())
             if swiglu:
                 return ops.swiglu(prod)
-            if residual is not None:
-                return ops.add(prod, residual.contiguous())
             return prod.float() if out_f32 else prod
         out = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)
         return ops.swiglu(out) if swiglu else out
