@@ -30,10 +30,13 @@ ATTN_CASES = [
     ([1, 3], [1000, 515], 32, 8, 128, 16, 0),  # head size 128, many heads
     ([33, 1, 1], [200, 200, 31], 4, 2, 64, 16, 40),  # a window: far keys must not be read
     ([5], [77], 20, 1, 16, 4, 0),  # group of 20: more rows of one token than a tile
+    ([300], [300], 8, 2, 64, 16, 0),  # a long prompt: 75 row tiles, an odd number to pair
+    ([257, 3, 1], [400, 50, 333], 4, 1, 64, 64, 100),  # pages of 64, a window shorter than the portion
+    ([90], [1000], 4, 2, 80, 32, 0),  # a portion far into a request, pages of 32, head size 80
 ]
 
 
-def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1, waves=1):
+def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1, waves=1, pair=False):
     from tokasaurus_amd.kernels import ops
 
     dtype = torch.bfloat16 if kind != "generic_f32" else torch.float32
@@ -44,28 +47,36 @@ def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=N
         token_req = torch.tensor([r for r, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32).cuda()
         positions = torch.tensor([kv - ql + j for ql, kv in zip(q_lens, kv_lens) for j in range(ql)], dtype=torch.int32).cuda()
         return ops.paged_attention_generic(q, kc, vc, table, token_req, positions, nq, nkv, d, page, window=window)
-    tile_req, tile_row0 = ops.attention_tiles(q_lens, nq // nkv, row_tiles)
+    tile_req, tile_row0, tile_row1 = ops.attention_tiles(q_lens, nq // nkv, row_tiles, pair=pair)
     max_kv = max(kv_lens)
     if split is None:
-        split, waves = ops.attention_split(max_kv, len(tile_req), nkv)
+        split, waves = ops.attention_split(max_kv, len(tile_req), nkv, d)
     return ops.paged_attention_mfma(
         q, kc, vc, table, dev(case["q_start"]), dev(case["kv_len"]),
         torch.tensor(tile_req, dtype=torch.int32).cuda(), torch.tensor(tile_row0, dtype=torch.int32).cuda(),
         row_tiles, nq, nkv, d, page, max_kv, split, window=window, waves=waves,
+        tile_row1=None if tile_row1 is None else torch.tensor(tile_row1, dtype=torch.int32).cuda(),
     )
 
 
 @pytest.mark.parametrize("case_id", range(len(ATTN_CASES)))
-@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma", "mfma_split32", "mfma_rt2", "mfma_waves4", "mfma_waves16"])
+@pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma", "mfma_split32", "mfma_rt2", "mfma_rt2_waves4",
+                                  "mfma_pairs", "mfma_pairs_split32", "mfma_waves4", "mfma_waves16"])
 def test_paged_attention(kind, case_id):
     q_lens, kv_lens, nq, nkv, d, page, window = ATTN_CASES[case_id]
     dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
     case = make_paged_case(q_lens, kv_lens, nq, nkv, d, page, seed=case_id, dtype=dtype)
     ref = attention_reference(case, q_lens, kv_lens, nq, nkv, d, window=window)
-    split = {"mfma_split32": 32, "mfma_rt2": 64, "mfma_waves4": 256, "mfma_waves16": 512}.get(kind)
-    waves = {"mfma_waves4": 4, "mfma_waves16": 16}.get(kind, 1)
+    split = {"mfma_split32": 32, "mfma_rt2": 64, "mfma_rt2_waves4": 128, "mfma_pairs": 4096, "mfma_pairs_split32": 32,
+             "mfma_waves4": 256, "mfma_waves16": 512}.get(kind)
+    waves = {"mfma_waves4": 4, "mfma_rt2_waves4": 4, "mfma_waves16": 16}.get(kind, 1)
+    two = kind in ("mfma_rt2", "mfma_rt2_waves4", "mfma_pairs", "mfma_pairs_split32")
+    if kind.startswith("mfma"):
+        from tokasaurus_amd.kernels import ops
+
+        waves = min(waves, ops.attention_max_waves(d, 2 if two else 1))  # head sizes above 64 take 8 at most
     got = run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=split,
-                        row_tiles=2 if kind == "mfma_rt2" else 1, waves=waves).float().cpu()
+                        row_tiles=2 if two else 1, waves=waves, pair="pairs" in kind).float().cpu()
     assert torch.isfinite(got).all()
     # values are of order 1; bfloat16 rounds the probabilities and the output to 8 bits
     tol = dict(atol=2e-5, rtol=1e-4) if kind == "generic_f32" else dict(atol=2e-2, rtol=2e-2)

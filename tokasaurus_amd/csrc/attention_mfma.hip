@@ -2,10 +2,10 @@
 // One kernel serves prompt portions and single decoded tokens.
 //
 // Rows.  For a request and a kv head, the rows are the pairs (token of this step,
-// query head of the kv head's group), numbered token * group + head.  A wavefront
-// owns RT tiles of 16 consecutive rows and walks the keys its rows may see in
-// steps of 32.  With the keys as the first operand of v_mfma_f32_16x16x32_bf16
-// and the queries as the second,
+// query head of the kv head's group), numbered token * group + head, and cut into
+// row tiles of 16.  A wavefront owns RT row tiles of one request and walks the keys
+// they may see in steps of 32.  With the keys as the first operand of
+// v_mfma_f32_16x16x32_bf16 and the queries as the second,
 //     S^T[key 4q+j][row r]  is element j of lane (r = lane % 16, q = lane / 16),
 // so a lane holds, for ONE row, 4 keys of each 16-key block.  These 8 numbers
 // are exactly what the lane must provide as the second operand of the product
@@ -14,10 +14,16 @@
 // pages are stored transposed ([d][P]), so the matching first operand is read
 // with two 8-byte loads per lane.  Nothing passes through LDS.
 //
-//   K pages: [page][kv head][P][d]      V pages: [page][kv head][d][P], P % 4 == 0
+//   K pages: [page][kv head][P][d]      V pages: [page][kv head][d][P]
+//   P a power of two, at least 4
 //
-// Splits.  The keys of a tile are cut at absolute multiples of `split`; each
-// (tile, kv head, split) is one workgroup of NW wavefronts, which cut the split's
+// Two row tiles of a wavefront need not be neighbours: under a causal mask the host
+// pairs an early tile of a prompt with a late one, so that every wavefront has the
+// same number of (row tile, key step) products.  A row tile is skipped in the steps
+// that none of its rows sees; steps that all of its rows see whole are not masked.
+//
+// Splits.  The keys of a wavefront's tiles are cut at absolute multiples of `split`;
+// each (tile, kv head, split) is one workgroup of NW wavefronts, which cut the split's
 // keys into NW consecutive parts (multiples of 32) and add their results through
 // LDS in wavefront order.  A tile with one split writes the output; otherwise
 // partial (max, sum, weighted values) go to scratch and a second kernel adds them
@@ -41,33 +47,54 @@ struct AttnArgs {
   const int* q_start;   // [requests + 1]
   const int* kv_len;    // [requests]
   const int* tile_req;  // [tiles]
-  const int* tile_row0; // [tiles]
+  const int* tile_row0; // [tiles] first row of the wavefront's first row tile
+  const int* tile_row1; // [tiles] first row of its second row tile, -1 for none; null: the 16 rows after the first
   int n_tiles;
-  int nq, nkv, group, P, window;
-  float scale;
-  int split;       // keys per split, a multiple of 32
-  int max_splits;  // splits a tile may have (size of the scratch)
-  float* part_o;   // [tiles][nkv][max_splits][16 * RT][D]
-  float* part_ml;  // [tiles][nkv][max_splits][16 * RT][2]
+  int nq, nkv, group, P, p_shift, window;
+  float scale_log2;  // scale * log2(e): scores are kept in units of log 2
+  int split;         // keys per split, a multiple of 32
+  int max_splits;    // splits a tile may have (size of the scratch)
+  float* part_o;     // [tiles][nkv][max_splits][16 * RT][D]
+  float* part_ml;    // [tiles][nkv][max_splits][16 * RT][2]
 };
 
+// What a (wavefront's) tile covers.  Per row tile: rows row0 .. row0 + 15 (row0 < 0: none),
+// keys [lo, hi] that some row sees and [full_lo, full_hi] that every row sees.
 struct TileRange {
-  int req, row0, qs, qlen, kvl, n_rows, lo, hi, s_first, s_last;
+  int req, qs, qlen, kvl, n_rows, lo, hi, s_first, s_last;
+  int row0[2], rt_lo[2], rt_hi[2], full_lo[2], full_hi[2];
 };
 
-__device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int rows_per_tile) {
+__device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int row_tiles) {
   TileRange t;
   t.req = a.tile_req[tile];
-  t.row0 = a.tile_row0[tile];
   t.qs = a.q_start[t.req];
   t.qlen = a.q_start[t.req + 1] - t.qs;
   t.kvl = a.kv_len[t.req];
   t.n_rows = t.qlen * a.group;
-  const int first_tok = t.row0 / a.group;
-  const int last_tok = min(t.row0 + rows_per_tile - 1, t.n_rows - 1) / a.group;
-  const int pos_first = t.kvl - t.qlen + first_tok;
-  t.hi = t.kvl - t.qlen + last_tok;
-  t.lo = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+  t.row0[0] = a.tile_row0[tile];
+  t.row0[1] = -1;
+  if (row_tiles == 2) {
+    t.row0[1] = a.tile_row1 ? a.tile_row1[tile] : t.row0[0] + 16;
+    if (t.row0[1] >= t.n_rows) t.row0[1] = -1;
+  }
+  t.lo = 0x7fffffff;
+  t.hi = -1;
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    t.rt_lo[rt] = t.full_lo[rt] = 0x7fffffff;
+    t.rt_hi[rt] = t.full_hi[rt] = -1;
+    if (t.row0[rt] < 0) continue;
+    const int first_tok = t.row0[rt] / a.group;
+    const int last_tok = min(t.row0[rt] + 15, t.n_rows - 1) / a.group;
+    const int pos_first = t.kvl - t.qlen + first_tok, pos_last = t.kvl - t.qlen + last_tok;
+    t.rt_hi[rt] = pos_last;
+    t.rt_lo[rt] = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+    t.full_hi[rt] = pos_first;
+    t.full_lo[rt] = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;
+    t.lo = min(t.lo, t.rt_lo[rt]);
+    t.hi = max(t.hi, t.rt_hi[rt]);
+  }
   t.s_first = t.lo / a.split;
   t.s_last = t.hi / a.split;
   return t;
@@ -75,25 +102,45 @@ __device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int
 
 // The loads of one step of 32 keys.  Keys: lane (r, q) reads 8 values of key
 // kb + 16 blk + r for every 32-wide step over the head size.  Values: lane (r, q)
-// reads, for d = 16 dt + r, the 4 keys kb + 16 blk + 4q .. + 3.  Addresses are
-// clamped into the tile's key range [lo, hi], so a load past the end reads valid memory.
+// reads, for d = 16 dt + r, the 4 keys kb + 16 blk + 4q .. + 3.  Every address lies
+// in a page of the tile's key range [lo, hi], so a load past the end reads valid
+// memory (whose contents the masks keep out of the result).
 template <int DT>
 struct StepRegs {
   bf16x8_t kv[2][(DT + 1) / 2];
-  bf16x4_t vv[DT][2];
+  union { bf16x4_t half[2]; uint32_t u[4]; bf16x8_t whole; } vv[DT];  // the two 16-key blocks side by side
 };
 
-template <int DT>
+// BIG: pages of 16 keys or more, so the 16 keys of a block lie in one page, which a
+// scalar load looks up; the lane's part of the address is the same in every step.
+template <int DT, bool BIG>
 __device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, const int* table,
                                           int kvh, int kb, int lo, int hi, int r, int q) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
-  const int P = a.P;
+  const int P = a.P, sh = a.p_shift;
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
-    const int kk = min(max(kb + blk * 16 + r, lo), hi);
-    const int page = table[kk / P];
-    const bf16_t* kp = a.kcache + ((size_t)((size_t)page * a.nkv + kvh) * P + (kk % P)) * D;
+    const bf16_t* kp;
+    const bf16_t* vp;
+    if constexpr (BIG) {
+      const int key0 = kb + blk * 16;
+      const int pidx = min(max(key0 >> sh, lo >> sh), hi >> sh);
+      const int page = table[pidx];
+      const size_t base = ((size_t)page * a.nkv + kvh) * ((size_t)P * D);
+      const int in_page = key0 & (P - 1);
+      kp = a.kcache + base + (size_t)in_page * D + r * D;
+      vp = a.vcache + base + in_page + r * P + q * 4;
+    } else {
+      const int kk = min(max(kb + blk * 16 + r, lo), hi);
+      const int page = table[kk >> sh];
+      kp = a.kcache + ((size_t)((size_t)page * a.nkv + kvh) * P + (kk & (P - 1))) * D;
+      int kc = kb + blk * 16 + q * 4;
+      if (kc > hi) kc = hi & ~3;
+      if (kc + 3 < lo) kc = lo & ~3;
+      const int vpage = table[kc >> sh];
+      vp = a.vcache + ((size_t)((size_t)vpage * a.nkv + kvh) * D + r) * P + (kc & (P - 1));
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 32 + q * 8;
@@ -104,26 +151,27 @@ __device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, co
         for (int e = 0; e < 8; ++e) s.kv[blk][ks][e] = (__bf16)0.f;
       }
     }
-    int kc = kb + blk * 16 + q * 4;
-    if (kc > hi) kc = hi & ~3;
-    if (kc + 3 < lo) kc = lo & ~3;
-    const int vpage = table[kc / P];
-    const bf16_t* vp = a.vcache + ((size_t)((size_t)vpage * a.nkv + kvh) * D + r) * P + (kc % P);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) s.vv[dt][blk] = *(const bf16x4_t*)(vp + (size_t)dt * 16 * P);
+    for (int dt = 0; dt < DT; ++dt) s.vv[dt].half[blk] = *(const bf16x4_t*)(vp + (size_t)dt * 16 * P);
   }
 }
 
-template <int DT, int RT>
-__global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) {
+// Wavefronts a workgroup may have: the fewer, the more registers each has for loads in flight.
+__host__ __device__ constexpr int max_waves(int dt, int rt) { return rt == 2 ? 4 : (dt <= 4 ? 16 : 8); }
+
+// PF steps of loads are in flight: a lone wavefront on a long tile waits on memory otherwise.
+template <int DT, int RT, bool BIG>
+__global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_kernel(AttnArgs a) {
   extern __shared__ __align__(16) float wg_part[];  // [wavefront][16 * RT rows][D + 4], when NW > 1
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head size
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int PF = RT == 1 ? 2 : 3;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int NW = blockDim.x >> 6;
   const int r = lane & 15, q = lane >> 4;
   const int tile = blockIdx.x, kvh = blockIdx.y;
-  const TileRange t = tile_range(a, tile, 16 * RT);
+  const TileRange t = tile_range(a, tile, RT);
   const int s = t.s_first + blockIdx.z;
   if (s > t.s_last) return;
   const int nsp = t.s_last - t.s_first + 1;
@@ -132,15 +180,15 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
   const int k_begin = max((t.lo >> 5) << 5, s * a.split + wave * sub);
   const int k_end = min(t.hi + 1, s * a.split + (wave + 1) * sub);
   const int* table = a.block_table + (size_t)t.req * a.table_stride;
-  const int P = a.P;
 
   // this lane's row in each of the RT tiles
-  int pos_r[RT], lo_r[RT];
+  int pos_r[RT], lo_r[RT], flat_r[RT];
   bf16x8_t qv[RT][KS];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int flat = t.row0 + rt * 16 + r;
+    const int flat = t.row0[rt] >= 0 ? t.row0[rt] + r : t.n_rows;
     const bool valid = flat < t.n_rows;
+    flat_r[rt] = valid ? flat : -1;
     const int fl = valid ? flat : t.n_rows - 1;
     const int tok = fl / a.group, g = fl - tok * a.group;
     const int pos = t.kvl - t.qlen + tok;
@@ -159,7 +207,7 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
     }
   }
 
-  float m_run[RT], l_run[RT];
+  float m_run[RT], l_run[RT];  // running maximum (in units of log 2) and sum of this lane's keys
   f32x4_t acc[RT][DT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -169,40 +217,28 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
     for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  StepRegs<DT> cur;
-  if (k_begin < k_end) load_step<DT>(cur, a, table, kvh, k_begin, t.lo, t.hi, r, q);
-  for (int kb = k_begin; kb < k_end; kb += 32) {
-    // the next step's loads are in flight while this step is computed
-    StepRegs<DT> nxt;
-    load_step<DT>(nxt, a, table, kvh, kb + 32 < k_end ? kb + 32 : kb, t.lo, t.hi, r, q);
-
-    // values of keys outside the tile's range may be anything (a freed page): make them
-    // zero by masking their 16 bits
-    bf16x8_t vv[DT];
-    uint32_t keep[2][2];
+  auto compute_step = [&](StepRegs<DT>& cur, const int kb) {
+    if (kb < t.lo || kb + 31 > t.hi) {
+      // values of keys outside the tile's range may be anything (a freed page): make them
+      // zero by masking their 16 bits
+      uint32_t keep[4];
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
+      for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int key = kb + blk * 16 + q * 4 + 2 * h;
-        const uint32_t lo16 = (key >= t.lo && key <= t.hi) ? 0x0000ffffu : 0u;
-        const uint32_t hi16 = (key + 1 >= t.lo && key + 1 <= t.hi) ? 0xffff0000u : 0u;
-        keep[blk][h] = lo16 | hi16;
-      }
+        for (int h = 0; h < 2; ++h) {
+          const int key = kb + blk * 16 + q * 4 + 2 * h;
+          const uint32_t lo16 = (key >= t.lo && key <= t.hi) ? 0x0000ffffu : 0u;
+          const uint32_t hi16 = (key + 1 >= t.lo && key + 1 <= t.hi) ? 0xffff0000u : 0u;
+          keep[blk * 2 + h] = lo16 | hi16;
+        }
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      union { bf16x4_t v[2]; uint32_t u[4]; bf16x8_t w; } x;
-      x.v[0] = cur.vv[dt][0];
-      x.v[1] = cur.vv[dt][1];
-      x.u[0] &= keep[0][0];
-      x.u[1] &= keep[0][1];
-      x.u[2] &= keep[1][0];
-      x.u[3] &= keep[1][1];
-      vv[dt] = x.w;
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) cur.vv[dt].u[i] &= keep[i];
     }
-
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+      if (kb > t.rt_hi[rt] || kb + 31 < t.rt_lo[rt]) continue;  // none of the tile's rows sees these keys
       f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -210,39 +246,56 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
         st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[1][ks], qv[rt][ks], st[1], 0, 0, 0);
       }
       float sc[8];
-      float mx = -INFINITY;
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
+      for (int e = 0; e < 8; ++e) sc[e] = st[e >> 2][e & 3] * a.scale_log2;
+      if (kb < t.full_lo[rt] || kb + 31 > t.full_hi[rt]) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int key = kb + blk * 16 + q * 4 + j;
-          const bool seen = key >= lo_r[rt] && key <= pos_r[rt];
-          const float v = seen ? st[blk][j] * a.scale : -INFINITY;
-          sc[blk * 4 + j] = v;
-          mx = fmaxf(mx, v);
+        for (int e = 0; e < 8; ++e) {
+          const int key = kb + (e >> 2) * 16 + q * 4 + (e & 3);
+          if (!(key >= lo_r[rt] && key <= pos_r[rt])) sc[e] = -INFINITY;
         }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run[rt], mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __expf(m_run[rt] - m_use);  // exp(-inf) = 0 while nothing was seen
+      if (__any(m_new > m_run[rt])) {
+        // some row's maximum moved: weigh what was summed so far
+        const float alpha = exp2f(m_run[rt] - m_use);  // exp2(-inf) = 0 while nothing was seen
+        l_run[rt] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[rt][dt] *= alpha;
+        m_run[rt] = m_new;
+      }
       float psum = 0.f;
       bf16x8_t pb;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = __expf(sc[e] - m_use);
+        const float p = exp2f(sc[e] - m_use);
         psum += p;
         pb[e] = (__bf16)p;
       }
-      m_run[rt] = m_new;
-      l_run[rt] = l_run[rt] * alpha + psum;
+      l_run[rt] += psum;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        acc[rt][dt] *= alpha;
-        acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[dt], pb, acc[rt][dt], 0, 0, 0);
+      for (int dt = 0; dt < DT; ++dt)
+        acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vv[dt].whole, pb, acc[rt][dt], 0, 0, 0);
+    }
+  };
+
+  StepRegs<DT> ring[PF];
+#pragma unroll
+  for (int i = 0; i < PF; ++i)
+    if (k_begin + 32 * i < k_end) load_step<DT, BIG>(ring[i], a, table, kvh, k_begin + 32 * i, t.lo, t.hi, r, q);
+  for (int kb = k_begin; kb < k_end; kb += 32 * PF) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int k = kb + 32 * i;
+      if (k < k_end) {
+        compute_step(ring[i], k);
+        if (k + 32 * PF < k_end) load_step<DT, BIG>(ring[i], a, table, kvh, k + 32 * PF, t.lo, t.hi, r, q);
       }
     }
-    cur = nxt;
   }
 
   // acc[rt][dt][j] of lane (r, q) is O^T[d = 16 dt + 4q + j][row r]
@@ -279,7 +332,7 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
       for (int w = 0; w < NW; ++w) {
         const float* row = wg_part + ((size_t)w * 16 * RT + rt * 16 + r) * ROW;
         const float mw = row[0];
-        const float f = (mw == -INFINITY) ? 0.f : __expf(mw - m);
+        const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - m);
         l += f * row[1];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[rt][dt] += f * *(const f32x4_t*)(row + 4 + dt * 16 + q * 4);
@@ -291,8 +344,8 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const float l = l_run[rt];
-    const int flat = t.row0 + rt * 16 + r;
-    if (flat >= t.n_rows) continue;
+    const int flat = flat_r[rt];
+    if (flat < 0) continue;
     if (nsp == 1) {
       const int tok = flat / a.group, g = flat - tok * a.group;
       bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
@@ -321,14 +374,17 @@ __global__ __launch_bounds__(1024) void paged_attention_mfma_kernel(AttnArgs a) 
 // Adds the partial results of split tiles, always in split order.  One wavefront
 // per (tile, kv head, row); lane i first takes the statistics of split i, then
 // every lane sums one (or more) of the row's d outputs over the splits.
-__global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D, int rows_per_tile) {
+__global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D, int row_tiles) {
   const int tile = blockIdx.x, kvh = blockIdx.y;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.z * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  const TileRange t = tile_range(a, tile, rows_per_tile);
+  const int rows_per_tile = 16 * row_tiles;
+  const TileRange t = tile_range(a, tile, row_tiles);
   const int nsp = t.s_last - t.s_first + 1;
   if (nsp == 1) return;
-  if (row >= min(rows_per_tile, t.n_rows - t.row0)) return;
+  const int base = t.row0[row >> 4];
+  const int flat = base + (row & 15);
+  if (base < 0 || flat >= t.n_rows) return;
   const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
   const float* ml = a.part_ml + (item0 * rows_per_tile + row) * 2;  // split sp is sp * rows_per_tile * 2 further
   const size_t ml_step = (size_t)rows_per_tile * 2;
@@ -338,11 +394,10 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D,
   float l = 0.f;
   for (int sp = lane; sp < nsp; sp += 64) {
     const float ms = ml[sp * ml_step];
-    l += (ms == -INFINITY ? 0.f : __expf(ms - m)) * ml[sp * ml_step + 1];
+    l += (ms == -INFINITY ? 0.f : exp2f(ms - m)) * ml[sp * ml_step + 1];
   }
   l = wave_sum(l);
   const float inv = 1.0f / l;
-  const int flat = t.row0 + row;
   const int tok = flat / a.group, g = flat - tok * a.group;
   bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
   const float* po = a.part_o + (item0 * rows_per_tile + row) * D;
@@ -352,7 +407,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D,
 #pragma unroll 8
     for (int sp = 0; sp < nsp; ++sp) {
       const float ms = ml[sp * ml_step];
-      const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
+      const float w = ms == -INFINITY ? 0.f : exp2f(ms - m);
       o += w * po[sp * po_step + d];
     }
     op[d] = __float2bfloat16(o * inv);
@@ -362,7 +417,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D,
 template <int DT, int RT>
 static bool launch_attn(const AttnArgs& a, int grid_splits, int nw, hipStream_t stream) {
   const size_t lds = nw > 1 ? (size_t)nw * 16 * RT * (DT * 16 + 4) * sizeof(float) : 0;
-  auto kernel = paged_attention_mfma_kernel<DT, RT>;
+  auto kernel = a.P >= 16 ? paged_attention_mfma_kernel<DT, RT, true> : paged_attention_mfma_kernel<DT, RT, false>;
   if (lds > 64 * 1024 &&
       hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return false;
@@ -385,27 +440,31 @@ static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, int nw, hi
   }
 }
 
-// Rows per tile are 16 * row_tiles (1 or 2); `waves` wavefronts share a split.  `tile_req`/`tile_row0` list the
-// tiles; `grid_splits` is an upper bound on the splits of any tile and
-// `max_splits` the number the scratch has room for (grid_splits <= max_splits).
-// part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
-// tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when max_splits
-// is 1).  Launches that share scratch must not overlap.
+// A wavefront owns row_tiles (1 or 2) tiles of 16 rows of one request: the rows from
+// tile_row0[i] and, with two, the rows from tile_row1[i] (-1: none; a null tile_row1: the
+// 16 rows after the first tile).  `waves` wavefronts share a split (at most 16; 8 with a
+// head size above 64; 4 with two row tiles).  `grid_splits` is an upper bound on the
+// splits of any tile and `max_splits` the number the scratch has room for (grid_splits <=
+// max_splits).  part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
+// tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when max_splits is 1).
+// Launches that share scratch must not overlap.
 TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                                        const void* kcache, const void* vcache,
                                        const int* block_table, int table_stride,
                                        const int* q_start, const int* kv_len,
-                                       const int* tile_req, const int* tile_row0, int n_tiles,
-                                       int row_tiles, int nq, int nkv, int d, int P, int window,
+                                       const int* tile_req, const int* tile_row0, const int* tile_row1,
+                                       int n_tiles, int row_tiles, int nq, int nkv, int d, int P, int window,
                                        float scale, int split, int waves, int grid_splits, int max_splits,
                                        float* part_o, float* part_ml, hipStream_t stream) {
   TK_REQUIRE(n_tiles >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_mfma: bad sizes tiles=%d nq=%d nkv=%d", n_tiles, nq, nkv);
   TK_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attention_mfma: head size %d is not a multiple of 16 up to 128", d);
-  TK_REQUIRE(P > 0 && P % 4 == 0, "attention_mfma: page size %d is not a multiple of 4", P);
+  TK_REQUIRE(P >= 4 && (P & (P - 1)) == 0, "attention_mfma: page size %d is not a power of two from 4", P);
   TK_REQUIRE(row_tiles == 1 || row_tiles == 2, "attention_mfma: row_tiles %d outside 1..2", row_tiles);
+  TK_REQUIRE(row_tiles == 2 || !tile_row1, "attention_mfma: second row tiles given with one row tile a wavefront");
   TK_REQUIRE(split > 0 && split % 32 == 0, "attention_mfma: split %d is not a multiple of 32", split);
-  TK_REQUIRE(waves >= 1 && waves <= 16 && split % (32 * waves) == 0,
-             "attention_mfma: %d wavefronts do not cut a split of %d keys into multiples of 32", waves, split);
+  TK_REQUIRE(waves >= 1 && waves <= max_waves(d / 16, row_tiles) && split % (32 * waves) == 0,
+             "attention_mfma: %d wavefronts (at most %d) do not cut a split of %d keys into multiples of 32", waves,
+             max_waves(d / 16, row_tiles), split);
   TK_REQUIRE((size_t)waves * 16 * row_tiles * (d + 4) * sizeof(float) <= 160 * 1024 || waves == 1,
              "attention_mfma: %d wavefronts of head size %d do not fit the local memory", waves, d);
   TK_REQUIRE(grid_splits >= 1 && grid_splits <= max_splits && grid_splits < 65536, "attention_mfma: splits %d of %d", grid_splits, max_splits);
@@ -420,8 +479,11 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
   a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
   a.kcache = (const bf16_t*)kcache; a.vcache = (const bf16_t*)vcache;
   a.block_table = block_table; a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len;
-  a.tile_req = tile_req; a.tile_row0 = tile_row0; a.n_tiles = n_tiles;
-  a.nq = nq; a.nkv = nkv; a.group = nq / nkv; a.P = P; a.window = window; a.scale = scale;
+  a.tile_req = tile_req; a.tile_row0 = tile_row0; a.tile_row1 = tile_row1; a.n_tiles = n_tiles;
+  a.nq = nq; a.nkv = nkv; a.group = nq / nkv; a.P = P; a.window = window;
+  a.p_shift = 0;
+  while ((1 << a.p_shift) < P) ++a.p_shift;
+  a.scale_log2 = scale * 1.4426950408889634f;
   a.split = split; a.max_splits = max_splits; a.part_o = part_o; a.part_ml = part_ml;
   const bool ok = row_tiles == 1 ? launch_attn_d<1>(a, d / 16, grid_splits, waves, stream)
                                  : launch_attn_d<2>(a, d / 16, grid_splits, waves, stream);
@@ -429,7 +491,7 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
   TK_CHECK_LAUNCH("paged_attention_mfma");
   if (max_splits > 1) {
     const int rows = 16 * row_tiles;
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_tiles, nkv, rows / 4), dim3(256), 0, stream, a, d, rows);
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_tiles, nkv, rows / 4), dim3(256), 0, stream, a, d, row_tiles);
     TK_CHECK_LAUNCH("attention_merge");
   }
   return 0;

@@ -300,33 +300,54 @@ def paged_attention_generic(
 
 def attention_mfma_supports(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
     """Whether the matrix-core attention kernel takes this storage type, head size and page size."""
-    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128 and page_size % 4 == 0
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128
+            and page_size >= 4 and page_size & (page_size - 1) == 0)
 
 
-def attention_tiles(q_lens: list[int], group: int, row_tiles: int) -> tuple[list[int], list[int]]:
-    """The tiles of 16 * row_tiles rows that cover every request's (token, head of the group) pairs."""
-    rows = 16 * row_tiles
+def attention_tiles(
+    q_lens: list[int], group: int, row_tiles: int, requests: list[int] | None = None, pair: bool = False
+) -> tuple[list[int], list[int], list[int] | None]:
+    """The row tiles that cover the (token, head of the group) pairs of ``requests``
+    (all by default), ``row_tiles`` tiles of 16 rows a wavefront: (request, first row of
+    the first tile, first row of the second tile or -1).  With ``pair`` a request's
+    i-th tile shares a wavefront with its i-th last, which evens out the keys a
+    wavefront walks under a causal mask; otherwise with its neighbour, and the
+    third list is None."""
     tile_req: list[int] = []
     tile_row0: list[int] = []
-    for r, n in enumerate(q_lens):
-        for row0 in range(0, n * group, rows):
+    tile_row1: list[int] = []
+    for r in (range(len(q_lens)) if requests is None else requests):
+        n = -(-q_lens[r] * group // 16)  # row tiles of the request
+        if row_tiles == 1:
+            firsts = [(i, -1) for i in range(n)]
+        elif pair:
+            firsts = [(i, n - 1 - i if n - 1 - i > i else -1) for i in range((n + 1) // 2)]
+        else:
+            firsts = [(i, i + 1 if i + 1 < n else -1) for i in range(0, n, 2)]
+        for i, j in firsts:
             tile_req.append(r)
-            tile_row0.append(row0)
-    return tile_req, tile_row0
+            tile_row0.append(16 * i)
+            tile_row1.append(16 * j if j >= 0 else -1)
+    return tile_req, tile_row0, (tile_row1 if pair and row_tiles == 2 else None)
 
 
-def attention_split(max_kv_len: int, n_tiles: int, nkv: int) -> tuple[int, int]:
-    """(keys per split, wavefronts per workgroup).  With few tiles (decode) the keys are
-    cut so that about four thousand wavefronts share the work, each with 64 to 512
-    keys, 4 to 16 of them a workgroup (measured best on an MI355X at 8192 keys:
-    64 keys x 4 at batch 1, 128 x 8 at batch 8, 512 x 16 at batch 64); with thousands
-    of tiles (prompts) nothing is split and a workgroup is one wavefront."""
+def attention_max_waves(head_dim: int, row_tiles: int) -> int:
+    """Wavefronts a workgroup of the matrix-core attention may have."""
+    return 4 if row_tiles == 2 else (16 if head_dim <= 64 else 8)
+
+
+def attention_split(max_kv_len: int, n_tiles: int, nkv: int, head_dim: int = 64) -> tuple[int, int]:
+    """(keys per split, wavefronts per workgroup) for tiles of one row tile.  With few
+    tiles (decode) the keys are cut so that about four thousand wavefronts share the
+    work, each with 64 to 512 keys, 4 to 16 of them a workgroup (measured best on an
+    MI355X at 8192 keys: 64 keys x 4 at batch 1, 128 x 8 at batch 8, 512 x 16 at batch
+    64); with thousands of tiles nothing is split and a workgroup is one wavefront."""
     base = max(n_tiles * nkv, 1)
     whole = -(-max(max_kv_len, 1) // 128) * 128
     if base >= 2048:
         return whole, 1
     sub = min(512, max(64, -(-(max_kv_len * base // 4096) // 32) * 32))
-    waves = 4 if base <= 16 else (8 if base <= 128 else 16)
+    waves = min(4 if base <= 16 else (8 if base <= 128 else 16), attention_max_waves(head_dim, 1))
     return sub * waves, waves
 
 
@@ -377,12 +398,15 @@ def paged_attention_mfma(
     waves: int = 1,
     out: torch.Tensor | None = None,
     scratch: "AttentionScratch | None" = None,
+    tile_row1: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Attention of every token of the batch over its request's pages on the
     matrix cores (bfloat16).  ``q`` is 2-d and its first nq*d columns are the
     query heads; request r owns tokens q_start[r]..q_start[r+1]-1, the last of
     them at position kv_len[r]-1.  ``max_kv_len`` bounds kv_len (it sizes the
-    grid and the scratch, so it may be larger than any request's)."""
+    grid and the scratch, so it may be larger than any request's).  The tiles
+    (see ``attention_tiles``) may cover some of the requests only; rows of ``out``
+    that no tile covers are left as they are."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * head_dim and q.dtype == torch.bfloat16,
           "attention_mfma: q must be bfloat16, 2-d with unit inner stride and nq*d leading columns")
@@ -398,6 +422,10 @@ def paged_attention_mfma(
           "attention_mfma: block table narrower than the longest request")
     n_tiles = tile_req.numel()
     _need(tile_row0.numel() == n_tiles, "attention_mfma: tile lists differ in length")
+    if tile_row1 is not None:
+        _gpu(tile_row1)
+        _i32(tile_row1, "tile_row1")
+        _need(tile_row1.numel() == n_tiles and row_tiles == 2, "attention_mfma: second row tiles need row_tiles == 2 and one entry a tile")
     pages = kcache.shape[0]
     _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
           "attention_mfma: key pages must be contiguous [pages, nkv, P, d]")
@@ -407,8 +435,9 @@ def paged_attention_mfma(
     _need(attention_mfma_supports(q.dtype, head_dim, page_size),
           f"attention_mfma: head size {head_dim} / page size {page_size} not supported")
     _need(split > 0 and split % 32 == 0, "attention_mfma: split must be a positive multiple of 32")
-    _need(1 <= waves <= 16 and split % (32 * waves) == 0,
-          "attention_mfma: the wavefronts of a workgroup must cut a split into multiples of 32 keys")
+    _need(1 <= waves <= attention_max_waves(head_dim, row_tiles) and split % (32 * waves) == 0,
+          "attention_mfma: the wavefronts of a workgroup (at most 16; 8 with a head size above 64; 4 with two row tiles) "
+          "must cut a split into multiples of 32 keys")
     if out is None:
         out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
     else:
@@ -425,6 +454,7 @@ def paged_attention_mfma(
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
         kcache.data_ptr(), vcache.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         q_start.data_ptr(), kv_len.data_ptr(), tile_req.data_ptr(), tile_row0.data_ptr(),
+        tile_row1.data_ptr() if tile_row1 is not None else None,
         n_tiles, row_tiles, nq, nkv, head_dim, page_size, int(window),
         float(scale if scale is not None else 1.0 / math.sqrt(head_dim)),
         split, waves, max_splits, max_splits,

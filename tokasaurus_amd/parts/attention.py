@@ -31,31 +31,59 @@ from tokasaurus_amd.parts.linear import Linear, Placer
 
 
 @dataclass
-class AttentionPlan:
-    """How the step's rows are cut into tiles and its keys into splits; made once
-    a step for each group size and shared by the layers."""
+class AttentionLaunch:
+    """One call of the matrix-core kernel: the tiles of some of the step's requests."""
 
     tile_req: torch.Tensor
     tile_row0: torch.Tensor
+    tile_row1: torch.Tensor | None
     row_tiles: int
-    max_kv_len: int
     split: int
     waves: int
     scratch: ops.AttentionScratch | None = None  # a replayed step keeps its own
 
 
-def attention_plan(ctx: StepContext, group: int, nkv: int) -> AttentionPlan:
-    key = ("attention_plan", group, nkv)
+@dataclass
+class AttentionPlan:
+    """How the step's rows are cut into tiles and its keys into splits; made once
+    a step for each group size and shared by the layers.  Requests that bring one
+    row tile or less (decoded tokens) get wavefronts of one row tile and split keys;
+    prompt portions get wavefronts of two row tiles, an early one paired with a late
+    one, and whole keys."""
+
+    launches: list[AttentionLaunch]
+    max_kv_len: int
+
+
+def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int) -> AttentionPlan:
+    key = ("attention_plan", group, nkv, head_dim)
     plan = ctx.extras.get(key)
     if plan is None:
         q_lens = [ctx.host_q_start[i + 1] - ctx.host_q_start[i] for i in range(ctx.num_requests)]
-        row_tiles = 2 if ctx.max_q_len * group > 16 else 1
-        tile_req, tile_row0 = ops.attention_tiles(q_lens, group, row_tiles)
-        tiles = torch.tensor([tile_req, tile_row0], dtype=torch.int32).to(ctx.device)
-        split, waves = ops.attention_split(ctx.max_kv_len, len(tile_req), nkv)
-        plan = AttentionPlan(tiles[0], tiles[1], row_tiles, ctx.max_kv_len, split, waves)
-        if ctx.extras.get("static"):
-            plan.scratch = ops.AttentionScratch(ctx.device)
+        small = [r for r, n in enumerate(q_lens) if 0 < n * group <= 16]
+        large = [r for r, n in enumerate(q_lens) if n * group > 16]
+        static = bool(ctx.extras.get("static"))
+        lists: list[tuple[list[int], list[int], list[int] | None, int, int, int]] = []
+        if small:
+            req, row0, _ = ops.attention_tiles(q_lens, group, 1, small)
+            split, waves = ops.attention_split(ctx.max_kv_len, len(req), nkv, head_dim)
+            lists.append((req, row0, None, 1, split, waves))
+        if large:
+            req, row0, row1 = ops.attention_tiles(q_lens, group, 2, large, pair=True)
+            whole = -(-max(ctx.max_kv_len, 1) // 128) * 128
+            lists.append((req, row0, row1, 2, whole, 1))
+        # one upload for all the tile lists of the step
+        flat = [x for req, row0, row1, *_ in lists for x in (req + row0 + (row1 or []))]
+        dev = torch.tensor(flat, dtype=torch.int32).to(ctx.device) if flat else None
+        launches, at = [], 0
+        for req, row0, row1, row_tiles, split, waves in lists:
+            n = len(req)
+            t_req, t_row0 = dev[at : at + n], dev[at + n : at + 2 * n]
+            t_row1 = dev[at + 2 * n : at + 3 * n] if row1 is not None else None
+            at += (3 if row1 is not None else 2) * n
+            launches.append(AttentionLaunch(t_req, t_row0, t_row1, row_tiles, split, waves,
+                                            ops.AttentionScratch(ctx.device) if static else None))
+        plan = AttentionPlan(launches, ctx.max_kv_len)
         ctx.extras[key] = plan
     return plan
 
@@ -134,12 +162,15 @@ class PagedAttention(Mixer):
                 cache.keys, cache.values, nq, nkv, d, cache.page_size, write_cache=cache.writable,
             )
         if ops.attention_mfma_supports(q.dtype, d, cache.page_size):
-            plan = attention_plan(ctx, nq // nkv, nkv)
-            attn = ops.paged_attention_mfma(
-                q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
-                plan.tile_req, plan.tile_row0, plan.row_tiles, nq, nkv, d, cache.page_size,
-                plan.max_kv_len, plan.split, window=self.window, scale=self.scale, waves=plan.waves, scratch=plan.scratch,
-            )
+            plan = attention_plan(ctx, nq // nkv, nkv, d)
+            attn = torch.empty((q.shape[0], nq * d), dtype=q.dtype, device=q.device)
+            for launch in plan.launches:
+                ops.paged_attention_mfma(
+                    q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
+                    launch.tile_req, launch.tile_row0, launch.row_tiles, nq, nkv, d, cache.page_size,
+                    plan.max_kv_len, launch.split, window=self.window, scale=self.scale, waves=launch.waves,
+                    out=attn, scratch=launch.scratch, tile_row1=launch.tile_row1,
+                )
         else:
             # the true 32-bit path, and shapes the matrix-core kernel does not take
             attn = ops.paged_attention_generic(
