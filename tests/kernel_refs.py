@@ -8,6 +8,28 @@ import math
 import torch
 
 
+def pack_key_pages(k: torch.Tensor) -> torch.Tensor:
+    """[pages, nkv, P, d] -> the engine's key pages [pages, nkv, d / 8, P, 8]."""
+    pages, nkv, P, d = k.shape
+    return k.reshape(pages, nkv, P, d // 8, 8).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def unpack_key_pages(k: torch.Tensor) -> torch.Tensor:
+    pages, nkv, pieces, P, eight = k.shape
+    return k.permute(0, 1, 3, 2, 4).reshape(pages, nkv, P, pieces * eight)
+
+
+def pack_value_pages(v: torch.Tensor) -> torch.Tensor:
+    """[pages, nkv, d, P] -> the engine's value pages [pages, nkv, P / 4, d, 4]."""
+    pages, nkv, d, P = v.shape
+    return v.reshape(pages, nkv, d, P // 4, 4).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def unpack_value_pages(v: torch.Tensor) -> torch.Tensor:
+    pages, nkv, quads, d, four = v.shape
+    return v.permute(0, 1, 3, 2, 4).reshape(pages, nkv, d, quads * four)
+
+
 def make_paged_case(
     q_lens: list[int],
     kv_lens: list[int],
@@ -23,7 +45,7 @@ def make_paged_case(
 ):
     """A batch of requests with shuffled pages.  Returns host tensors:
     q [N, nq*d], dense keys/values per request, the paged caches
-    (K [pages, nkv, P, d], V [pages, nkv, d, P]), block table, q_start, kv_len.
+    (packed as the engine keeps them), block table, q_start, kv_len.
     Queries are scaled so that scores have a spread of about ``sharp``: a
     missing or misplaced key then moves the result far beyond rounding.
     Unused cache entries are NaN when ``poison`` (nothing stale may be read)."""
@@ -58,8 +80,8 @@ def make_paged_case(
         "q": torch.cat(qs, 0),
         "k": dense_k,
         "v": dense_v,
-        "kcache": kc,
-        "vcache": vc,
+        "kcache": pack_key_pages(kc),
+        "vcache": pack_value_pages(vc),
         "table": table,
         "q_start": q_start,
         "kv_len": torch.tensor(kv_lens, dtype=torch.int32),

@@ -5,7 +5,7 @@ import math
 import pytest
 import torch
 
-from kernel_refs import attention_reference, make_paged_case
+from kernel_refs import attention_reference, make_paged_case, unpack_key_pages, unpack_value_pages
 
 pytestmark = pytest.mark.gpu
 
@@ -263,8 +263,8 @@ def test_gemm_rotation_with_append_epilogue(m, shape):
     sin = torch.sin(torch.arange(100)[:, None] * (10000.0 ** -inv)[None, :]).contiguous().cuda()
     caches = []
     for fused in (False, True):
-        kc = torch.full((m * width, nkv, page, d), 7.0, dtype=torch.bfloat16).cuda()
-        vc = torch.full((m * width, nkv, d, page), 7.0, dtype=torch.bfloat16).cuda()
+        kc = torch.full(ops.key_pages_shape(m * width, nkv, page, d), 7.0, dtype=torch.bfloat16).cuda()
+        vc = torch.full(ops.value_pages_shape(m * width, nkv, page, d), 7.0, dtype=torch.bfloat16).cuda()
         if fused:
             for tile_rows in (8, 16):
                 rope = ops.RopeAppend(positions.cuda(), token_req.cuda(), table.cuda(), cos, sin, kc, vc, nq, nkv, d, page)
@@ -395,8 +395,8 @@ def test_rope_append(dtype, shape):
         at += b
     inv = plain_llama.rope_inverse_frequencies(d, 10000.0, None)
     cos_t, sin_t = plain_llama.rope_tables(torch.arange(64), inv)
-    kc = torch.full((pages, nkv, page, d), 7.0).to(DT[dtype]).cuda()
-    vc = torch.full((pages, nkv, d, page), 7.0).to(DT[dtype]).cuda()
+    kc = torch.full(ops.key_pages_shape(pages, nkv, page, d), 7.0).to(DT[dtype]).cuda()
+    vc = torch.full(ops.value_pages_shape(pages, nkv, page, d), 7.0).to(DT[dtype]).cuda()
     dev_qkv = qkv.cuda()
     ops.rope_append(dev_qkv, positions.cuda(), token_req.cuda(), table.cuda(), cos_t[:, : d // 2].contiguous().cuda(),
                     sin_t[:, : d // 2].contiguous().cuda(), kc, vc, nq, nkv, d, page)
@@ -410,7 +410,7 @@ def test_rope_append(dtype, shape):
     tol = dict(atol=1e-6, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=1e-2)
     assert torch.allclose(out[:, : nq * d].view(n, nq, d).float(), want_q.float(), **tol)
     assert torch.equal(out[:, nq * d :], qkv[:, nq * d :]), "k and v columns of the input must stay as they were"
-    kc, vc = kc.cpu(), vc.cpu()
+    kc, vc = unpack_key_pages(kc.cpu()), unpack_value_pages(vc.cpu())  # [pages, nkv, P, d] and [pages, nkv, d, P]
     written = torch.zeros((pages, page), dtype=torch.bool)
     for t in range(n):
         p, o = int(table[token_req[t], positions[t] // page]), int(positions[t]) % page
@@ -455,9 +455,15 @@ def test_kernels_refuse_what_they_cannot_do():
     assert not ops.attention_mfma_supports(torch.bfloat16, 40, 16)
     assert not ops.attention_mfma_supports(torch.bfloat16, 64, 6)
     assert not ops.attention_mfma_supports(torch.float32, 64, 16)
-    # the generic attention takes any head size (here 40) and an odd page size
+    # the generic attention takes any head size that is a multiple of 8 (here 40) and a page
+    # size that is a multiple of 4 and no power of two
     q_lens, kv_lens = [3, 1], [11, 30]
-    case = make_paged_case(q_lens, kv_lens, 4, 2, 40, 6, seed=1, dtype=torch.float32)
+    case = make_paged_case(q_lens, kv_lens, 4, 2, 40, 12, seed=1, dtype=torch.float32)
     ref = attention_reference(case, q_lens, kv_lens, 4, 2, 40)
-    got = run_attention("generic_f32", case, q_lens, kv_lens, 4, 2, 40, 6, 0).cpu()
+    got = run_attention("generic_f32", case, q_lens, kv_lens, 4, 2, 40, 12, 0).cpu()
     assert torch.allclose(got, ref, atol=2e-5, rtol=1e-4)
+    assert not ops.attention_mfma_supports(torch.bfloat16, 64, 12)
+    with pytest.raises(KernelError, match="pieces of 8"):
+        ops.key_pages_shape(4, 2, 16, 20)
+    with pytest.raises(KernelError, match="groups of 4"):
+        ops.value_pages_shape(4, 2, 6, 64)

@@ -18,6 +18,7 @@ from test_replay_gpu import mixed_trace
 from tiny_models import CONFIG_A, CONFIG_B, random_tokens
 from tokasaurus_amd.engine.batch import PlannedEntry, layout, to_device
 from tokasaurus_amd.engine.runner import ModelRunner
+from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, CacheView, PartSpec
 from tokasaurus_amd.parts.block import stream_and_prepared
 from tokasaurus_amd.parts.embedding import LMHead, TokenEmbedding
@@ -144,8 +145,8 @@ def test_attention_mixer_and_block_alone(dtype, shape):
         need = (built if part == "mixer" else built.mixer).cache_need()
         assert (need.num_kv_heads, need.head_dim, need.window) == (nkv, d, window)
         pages = 32
-        keys = torch.full((pages, nkv, page, d), float("nan"), dtype=dt, device="cuda")
-        values = torch.full((pages, nkv, d, page), float("nan"), dtype=dt, device="cuda")
+        keys = torch.full(ops.key_pages_shape(pages, nkv, page, d), float("nan"), dtype=dt, device="cuda")
+        values = torch.full(ops.value_pages_shape(pages, nkv, page, d), float("nan"), dtype=dt, device="cuda")
         perm = torch.randperm(pages, generator=g).tolist()
         tab_a, tab_b = perm[: -(-lens["a"] // page)], perm[16 : 16 + -(-lens["b"] // page)]
         got = {}

@@ -1,10 +1,10 @@
 """Device tensors behind the cache manager's page ids and slots.
 
-Per group: keys ``[entries, pages, nkv, P, d]`` and values
-``[entries, pages, nkv, d, P]`` (values transposed inside a page, so that both
-the key rows of a page and the value columns of a page are contiguous for the
-attention kernels).  The reference keeps ``[pages, P, nkv, d]`` per layer for both
-(tokasaurus/model/kv_cache.py:27-54).  Per run entry with fixed-size state:
+Per group: keys ``[entries, pages, nkv, d / 8, P, 8]`` and values
+``[entries, pages, nkv, P / 4, d, 4]``: inside a page the keys lie in pieces of 8
+elements and the values in groups of 4 tokens, the order in which the lanes of the
+attention kernel read them (``kernels.ops.key_pages_shape``).  The reference keeps
+``[pages, P, nkv, d]`` per layer for both (tokasaurus/model/kv_cache.py:27-54).  Per run entry with fixed-size state:
 ``[slots + 1, *shape]``.  The last page of every pool and the last slot belong to
 no request: rows that only pad a step to a recorded size write there (the
 reference's scratch page, tokasaurus/model/utils.py:363-369,552-554).
@@ -15,6 +15,7 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.cache.manager import CacheGroup
+from tokasaurus_amd.kernels.ops import key_pages_shape, value_pages_shape
 from tokasaurus_amd.parts.base import StateNeed
 
 
@@ -35,8 +36,9 @@ class CacheStorage:
         for grp, n in zip(groups, num_pages):
             nkv, d = grp.need.num_kv_heads, grp.need.head_dim
             # one page more than the pool hands out: the null page, where padding rows write
-            self.keys.append(torch.zeros((len(grp.entries), n + 1, nkv, page_size, d), dtype=dtype, device=device))
-            self.values.append(torch.zeros((len(grp.entries), n + 1, nkv, d, page_size), dtype=dtype, device=device))
+            entries = (len(grp.entries),)
+            self.keys.append(torch.zeros(entries + key_pages_shape(n + 1, nkv, page_size, d), dtype=dtype, device=device))
+            self.values.append(torch.zeros(entries + value_pages_shape(n + 1, nkv, page_size, d), dtype=dtype, device=device))
         self.states: list[torch.Tensor | None] = [
             torch.zeros((max_slots + 1, *need.shape), dtype=need.dtype, device=device) if need is not None else None
             for need in state_needs

@@ -60,8 +60,9 @@ __global__ __launch_bounds__(AG_THREADS) void paged_attention_generic_kernel(
       if (kp >= lo && kp <= pos) {
         const int page = table[kp / P];
         const int p = kp % P;
-        kv = to_f32<T>(kcache[(((size_t)page * nkv + g) * P + p) * d + e]);
-        vv = to_f32<T>(vcache[(((size_t)page * nkv + g) * d + e) * P + p]);
+        const size_t base = ((size_t)page * nkv + g) * P * d;
+        kv = to_f32<T>(kcache[base + key_offset(P, p, e)]);
+        vv = to_f32<T>(vcache[base + value_offset(d, p, e)]);
       }
       Ks[j * (d + 1) + e] = kv;
       Vs[j * d + e] = vv;

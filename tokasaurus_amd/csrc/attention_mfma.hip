@@ -10,12 +10,13 @@
 // so a lane holds, for ONE row, 4 keys of each 16-key block.  These 8 numbers
 // are exactly what the lane must provide as the second operand of the product
 // O^T = V^T P^T, if slot 8q+j of that product's inner index stands for key 4q+j
-// of the first block and slot 8q+4+j for key 4q+j of the second.  The value
-// pages are stored transposed ([d][P]), so the matching first operand is read
-// with two 8-byte loads per lane.  Nothing passes through LDS.
-//
-//   K pages: [page][kv head][P][d]      V pages: [page][kv head][d][P]
-//   P a power of two, at least 4
+// of the first block and slot 8q+4+j for key 4q+j of the second.  A page keeps
+// its values in groups of 4 tokens ([P / 4][d][4]), so the matching first operand
+// is read with two 8-byte loads per lane, and its keys in pieces of 8 elements
+// ([d / 8][P][8]), so that in both kinds of load 16 neighbouring lanes read
+// consecutive memory: the vector cache handles a load at the rate of the cache
+// lines it touches, not of its bytes.  Nothing passes through LDS.
+// P is a power of two, at least 4.
 //
 // Two row tiles of a wavefront need not be neighbours: under a causal mask the host
 // pairs an early tile of a prompt with a late one, so that every wavefront has the
@@ -129,30 +130,30 @@ __device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, co
       const int page = table[pidx];
       const size_t base = ((size_t)page * a.nkv + kvh) * ((size_t)P * D);
       const int in_page = key0 & (P - 1);
-      kp = a.kcache + base + (size_t)in_page * D + r * D;
-      vp = a.vcache + base + in_page + r * P + q * 4;
+      kp = a.kcache + base + (size_t)(in_page + r) * 8;
+      vp = a.vcache + base + (size_t)(in_page >> 2) * (D * 4) + (size_t)(q * D + r) * 4;
     } else {
       const int kk = min(max(kb + blk * 16 + r, lo), hi);
       const int page = table[kk >> sh];
-      kp = a.kcache + ((size_t)((size_t)page * a.nkv + kvh) * P + (kk & (P - 1))) * D;
+      kp = a.kcache + ((size_t)page * a.nkv + kvh) * ((size_t)P * D) + (size_t)(kk & (P - 1)) * 8;
       int kc = kb + blk * 16 + q * 4;
       if (kc > hi) kc = hi & ~3;
       if (kc + 3 < lo) kc = lo & ~3;
       const int vpage = table[kc >> sh];
-      vp = a.vcache + ((size_t)((size_t)vpage * a.nkv + kvh) * D + r) * P + (kc & (P - 1));
+      vp = a.vcache + ((size_t)vpage * a.nkv + kvh) * ((size_t)P * D) + (size_t)((kc & (P - 1)) >> 2) * (D * 4) + r * 4;
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int d0 = ks * 32 + q * 8;
+      const int d0 = ks * 32 + q * 8;  // piece d0 / 8 of the key
       if (d0 < D) {
-        s.kv[blk][ks] = *(const bf16x8_t*)(kp + d0);
+        s.kv[blk][ks] = *(const bf16x8_t*)(kp + (size_t)(d0 >> 3) * P * 8);
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) s.kv[blk][ks][e] = (__bf16)0.f;
       }
     }
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) s.vv[dt].half[blk] = *(const bf16x4_t*)(vp + (size_t)dt * 16 * P);
+    for (int dt = 0; dt < DT; ++dt) s.vv[dt].half[blk] = *(const bf16x4_t*)(vp + dt * 64);
   }
 }
 

@@ -35,6 +35,20 @@ void tk_set_error(const char* fmt, ...);
     }                                                                        \
   } while (0)
 
+// Layout of a page of the cache (P tokens of one kv head, head size d), chosen so that
+// the lanes of a wavefront that feed the matrix cores read consecutive memory:
+//   keys   [d / 8][P][8]   the 8-element pieces of the P keys, piece by piece
+//   values [P / 4][d][4]   groups of 4 tokens, for each the d rows of 4 values
+// A page of kv head h of page `page` starts at ((page * nkv + h) * P * d).
+#define TK_KEY_PIECE 8
+#define TK_VALUE_QUAD 4
+__host__ __device__ __forceinline__ size_t key_offset(int P, int in_page, int e) {
+  return ((size_t)(e / TK_KEY_PIECE) * P + in_page) * TK_KEY_PIECE + (e % TK_KEY_PIECE);
+}
+__host__ __device__ __forceinline__ size_t value_offset(int d, int in_page, int e) {
+  return ((size_t)(in_page / TK_VALUE_QUAD) * d + e) * TK_VALUE_QUAD + (in_page % TK_VALUE_QUAD);
+}
+
 template <typename T>
 __device__ __forceinline__ float to_f32(T v);
 template <>

@@ -197,13 +197,13 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
     const int h = i / half, j = i % half;
     const float x1 = to_f32<T>(krow[h * d + j]), x2 = to_f32<T>(krow[h * d + j + half]);
     const float cj = c ? c[j] : 1.f, sj = s ? s[j] : 0.f;
-    T* dst = kcache + (((size_t)page * nkv + h) * P + p) * d;
-    dst[j] = from_f32<T>(x1 * cj - x2 * sj);
-    dst[j + half] = from_f32<T>(x2 * cj + x1 * sj);
+    T* dst = kcache + ((size_t)page * nkv + h) * P * d;
+    dst[key_offset(P, p, j)] = from_f32<T>(x1 * cj - x2 * sj);
+    dst[key_offset(P, p, j + half)] = from_f32<T>(x2 * cj + x1 * sj);
   }
   for (int i = threadIdx.x; i < nkv * d; i += blockDim.x) {
     const int h = i / d, e = i % d;
-    vcache[(((size_t)page * nkv + h) * d + e) * P + p] = vrow[i];
+    vcache[((size_t)page * nkv + h) * P * d + value_offset(d, p, e)] = vrow[i];
   }
 }
 

@@ -64,8 +64,8 @@ struct GemmArgs {
   int table_stride;
   const float* cos_t;  // [positions][d / 2], null: no rotation
   const float* sin_t;
-  bf16_t* kcache;  // [page][kv head][P][d]
-  bf16_t* vcache;  // [page][kv head][d][P]
+  bf16_t* kcache;  // [page][kv head] pages of keys
+  bf16_t* vcache;  // [page][kv head] pages of values
   int nq, nkv, d, P;
   int M, N, K;  // N: outputs (for SwiGLU the intermediate size; W then has 2N rows, gate first)
   int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
@@ -202,20 +202,20 @@ __device__ __forceinline__ void rope_store(const GemmArgs& a, f32x4_t s0, f32x4_
   const int page = a.block_table[(size_t)a.token_req[token] * a.table_stride + pos / a.P];
   const int off = pos % a.P;
   if (h < a.nq + a.nkv) {
-    bf16_t* dst = a.kcache + (((size_t)page * a.nkv + (h - a.nq)) * a.P + off) * a.d + c;
+    bf16_t* dst = a.kcache + ((size_t)page * a.nkv + (h - a.nq)) * a.P * a.d;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (c + j < half) {
-        dst[j] = __float2bfloat16(o1[j]);
-        dst[j + half] = __float2bfloat16(o2[j]);
+        dst[key_offset(a.P, off, c + j)] = __float2bfloat16(o1[j]);
+        dst[key_offset(a.P, off, c + j + half)] = __float2bfloat16(o2[j]);
       }
   } else {
-    bf16_t* dst = a.vcache + (((size_t)page * a.nkv + (h - a.nq - a.nkv)) * a.d + c) * a.P + off;
+    bf16_t* dst = a.vcache + ((size_t)page * a.nkv + (h - a.nq - a.nkv)) * a.P * a.d;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (c + j < half) {
-        dst[(size_t)j * a.P] = __float2bfloat16(o1[j]);
-        dst[(size_t)(j + half) * a.P] = __float2bfloat16(o2[j]);
+        dst[value_offset(a.d, off, c + j)] = __float2bfloat16(o1[j]);
+        dst[value_offset(a.d, off, c + j + half)] = __float2bfloat16(o2[j]);
       }
   }
 }

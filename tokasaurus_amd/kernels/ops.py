@@ -43,6 +43,34 @@ def _i32(t: torch.Tensor, name: str) -> None:
     _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
 
 
+KEY_PIECE = 8  # elements of a key that lie together in a page
+VALUE_QUAD = 4  # tokens whose values lie together in a page
+
+
+def key_pages_shape(pages: int, nkv: int, page_size: int, head_dim: int) -> tuple[int, ...]:
+    """Keys: [pages, nkv, d / 8, P, 8]: a page holds the 8-element pieces of its P
+    keys piece by piece, so that the lanes that feed the matrix cores (16 keys, one
+    piece each) read consecutive memory."""
+    _need(head_dim % KEY_PIECE == 0, f"the cache keeps keys in pieces of {KEY_PIECE}: head size {head_dim} is no multiple")
+    return (pages, nkv, head_dim // KEY_PIECE, page_size, KEY_PIECE)
+
+
+def value_pages_shape(pages: int, nkv: int, page_size: int, head_dim: int) -> tuple[int, ...]:
+    """Values: [pages, nkv, P / 4, d, 4]: a page holds its tokens in groups of 4,
+    for each group the d rows of 4 values."""
+    _need(page_size % VALUE_QUAD == 0, f"the cache keeps values in groups of {VALUE_QUAD} tokens: page size {page_size} is no multiple")
+    return (pages, nkv, page_size // VALUE_QUAD, head_dim, VALUE_QUAD)
+
+
+def _check_pages(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, page_size: int, head_dim: int, dtype: torch.dtype, who: str) -> None:
+    pages = kcache.shape[0]
+    _need(tuple(kcache.shape) == key_pages_shape(pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
+          f"{who}: key pages must be contiguous {key_pages_shape(pages, nkv, page_size, head_dim)}, got {tuple(kcache.shape)}")
+    _need(tuple(vcache.shape) == value_pages_shape(pages, nkv, page_size, head_dim) and vcache.is_contiguous(),
+          f"{who}: value pages must be contiguous {value_pages_shape(pages, nkv, page_size, head_dim)}, got {tuple(vcache.shape)}")
+    _need(kcache.dtype == dtype and vcache.dtype == dtype, f"{who}: the cache must be {dtype}")
+
+
 def embed_gather(
     ids: torch.Tensor, table: torch.Tensor, last_token: torch.Tensor | None = None
 ) -> torch.Tensor:
@@ -150,8 +178,8 @@ def rope_append(
     """Rotate the query heads of ``qkv`` in place; rotate the key heads and store
     them and the value heads in each token's page.
 
-    ``kcache`` is [pages, nkv, P, d], ``vcache`` is [pages, nkv, d, P] (values
-    transposed inside a page).  ``block_table`` is [requests, width] int32.
+    ``kcache`` and ``vcache`` have the shapes of ``key_pages_shape`` and
+    ``value_pages_shape``.  ``block_table`` is [requests, width] int32.
     """
     _gpu(qkv, positions, token_req, block_table, cos, sin, kcache, vcache)
     _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be 2-d with unit inner stride")
@@ -171,12 +199,7 @@ def rope_append(
         _i32(block_table, "block_table")
         _need(block_table.dim() == 2, "block_table must be [requests, width]")
         table_stride = block_table.stride(0)
-        pages = kcache.shape[0]
-        _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
-              f"key pages must be contiguous [pages, {nkv}, {page_size}, {head_dim}], got {tuple(kcache.shape)}")
-        _need(tuple(vcache.shape) == (pages, nkv, head_dim, page_size) and vcache.is_contiguous(),
-              f"value pages must be contiguous [pages, {nkv}, {head_dim}, {page_size}], got {tuple(vcache.shape)}")
-        _need(kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype, "cache dtype differs from qkv")
+        _check_pages(kcache, vcache, nkv, page_size, head_dim, qkv.dtype, "rope_append")
     call(
         "tk_rope_append",
         dtype_code(qkv.dtype),
@@ -266,12 +289,7 @@ def paged_attention_generic(
     _i32(positions, "positions")
     _need(block_table.dim() == 2, "block_table must be [requests, width]")
     _need(positions.numel() == n and token_req.numel() == n, "positions/token_req must have one entry a token")
-    pages = kcache.shape[0]
-    _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
-          "attention: key pages must be contiguous [pages, nkv, P, d]")
-    _need(tuple(vcache.shape) == (pages, nkv, head_dim, page_size) and vcache.is_contiguous(),
-          "attention: value pages must be contiguous [pages, nkv, d, P]")
-    _need(kcache.dtype == q.dtype and vcache.dtype == q.dtype, "attention: cache dtype differs from q")
+    _check_pages(kcache, vcache, nkv, page_size, head_dim, q.dtype, "attention")
     out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
     call(
         "tk_paged_attention_generic",
@@ -426,12 +444,7 @@ def paged_attention_mfma(
         _gpu(tile_row1)
         _i32(tile_row1, "tile_row1")
         _need(tile_row1.numel() == n_tiles and row_tiles == 2, "attention_mfma: second row tiles need row_tiles == 2 and one entry a tile")
-    pages = kcache.shape[0]
-    _need(tuple(kcache.shape) == (pages, nkv, page_size, head_dim) and kcache.is_contiguous(),
-          "attention_mfma: key pages must be contiguous [pages, nkv, P, d]")
-    _need(tuple(vcache.shape) == (pages, nkv, head_dim, page_size) and vcache.is_contiguous(),
-          "attention_mfma: value pages must be contiguous [pages, nkv, d, P]")
-    _need(kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16, "attention_mfma: the cache must be bfloat16")
+    _check_pages(kcache, vcache, nkv, page_size, head_dim, torch.bfloat16, "attention_mfma")
     _need(attention_mfma_supports(q.dtype, head_dim, page_size),
           f"attention_mfma: head size {head_dim} / page size {page_size} not supported")
     _need(split > 0 and split % 32 == 0, "attention_mfma: split must be a positive multiple of 32")
@@ -607,11 +620,7 @@ def gemm_skinny_bf16(
             _i32(t, name)
         _need(r.positions.numel() == m and r.token_req.numel() == m and r.block_table.dim() == 2,
               "gemm_skinny: positions/token_req need one entry a row, block_table [requests, width]")
-        pages = r.kcache.shape[0]
-        _need(tuple(r.kcache.shape) == (pages, r.nkv, r.page_size, r.head_dim) and r.kcache.is_contiguous()
-              and tuple(r.vcache.shape) == (pages, r.nkv, r.head_dim, r.page_size) and r.vcache.is_contiguous()
-              and r.kcache.dtype == torch.bfloat16 and r.vcache.dtype == torch.bfloat16,
-              "gemm_skinny: the pages must be contiguous bfloat16 [pages, nkv, P, d] and [pages, nkv, d, P]")
+        _check_pages(r.kcache, r.vcache, r.nkv, r.page_size, r.head_dim, torch.bfloat16, "gemm_skinny")
         if r.cos is not None:
             half = r.head_dim // 2
             _need(r.sin is not None and r.cos.dtype == torch.float32 and r.sin.dtype == torch.float32

@@ -73,8 +73,8 @@ class PartSpec:
 class CacheView:
     """The pages of one cache-owning run entry, and its group's block table for this step."""
 
-    keys: torch.Tensor  # [pages, nkv, P, d]
-    values: torch.Tensor  # [pages, nkv, d, P]
+    keys: torch.Tensor  # [pages, nkv, d / 8, P, 8]
+    values: torch.Tensor  # [pages, nkv, P / 4, d, 4]
     block_table: torch.Tensor  # [requests, width] int32, -1 where no page is held
     page_size: int
     writable: bool = True  # False when the entry reads another entry's cache
