@@ -33,6 +33,7 @@ ATTN_CASES = [
     ([300], [300], 8, 2, 64, 16, 0),  # a long prompt: 75 row tiles, an odd number to pair
     ([257, 3, 1], [400, 50, 333], 4, 1, 64, 64, 100),  # pages of 64, a window shorter than the portion
     ([90], [1000], 4, 2, 80, 32, 0),  # a portion far into a request, pages of 32, head size 80
+    ([1, 2], [2300, 40], 8, 2, 64, 16, 0),  # with splits of 32 keys: more splits (72) than a wavefront has lanes
 ]
 
 

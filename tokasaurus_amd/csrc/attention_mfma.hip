@@ -52,7 +52,7 @@ struct AttnArgs {
   const int* tile_row1; // [tiles] first row of its second row tile, -1 for none; null: the 16 rows after the first
   int n_tiles;
   int nq, nkv, group, P, p_shift, window;
-  float scale_log2;  // scale * log2(e): scores are kept in units of log 2
+  float scale_log2;  // scale * log2(e) > 0
   int split;         // keys per split, a multiple of 32
   int max_splits;    // splits a tile may have (size of the scratch)
   float* part_o;     // [tiles][nkv][max_splits][16 * RT][D]
@@ -99,6 +99,17 @@ __device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int
   t.s_first = t.lo / a.split;
   t.s_last = t.hi / a.split;
   return t;
+}
+
+// The maximum over the four lanes (r, 0..3) that share a row: lanes 16 and 32 apart,
+// with the gfx950 swaps of 16-lane rows and of wavefront halves.
+__device__ __forceinline__ float max_over_quarters(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const unsigned v = __float_as_uint(y);
+  const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
 // The loads of one step of 32 keys.  Keys: lane (r, q) reads 8 values of key
@@ -208,7 +219,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
     }
   }
 
-  float m_run[RT], l_run[RT];  // running maximum (in units of log 2) and sum of this lane's keys
+  float m_run[RT], l_run[RT];  // running maximum of the row's products and sum of this lane's keys
   f32x4_t acc[RT][DT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -246,9 +257,11 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
         st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[0][ks], qv[rt][ks], st[0], 0, 0, 0);
         st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[1][ks], qv[rt][ks], st[1], 0, 0, 0);
       }
+      // scores stay as the products are (scale_log2 > 0 keeps their order); the scale goes
+      // into the exponent's multiply-add
       float sc[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sc[e] = st[e >> 2][e & 3] * a.scale_log2;
+      for (int e = 0; e < 8; ++e) sc[e] = st[e >> 2][e & 3];
       if (kb < t.full_lo[rt] || kb + 31 > t.full_hi[rt]) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -257,13 +270,13 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
         }
       }
       float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_over_quarters(mx);
       const float m_new = fmaxf(m_run[rt], mx);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float mc = m_use * a.scale_log2;
       if (__any(m_new > m_run[rt])) {
         // some row's maximum moved: weigh what was summed so far
-        const float alpha = exp2f(m_run[rt] - m_use);  // exp2(-inf) = 0 while nothing was seen
+        const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run[rt], a.scale_log2, -mc));  // 0 while nothing was seen
         l_run[rt] *= alpha;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[rt][dt] *= alpha;
@@ -273,7 +286,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
       bf16x8_t pb;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = exp2f(sc[e] - m_use);
+        const float p = __builtin_amdgcn_exp2f(fmaf(sc[e], a.scale_log2, -mc));
         psum += p;
         pb[e] = (__bf16)p;
       }
@@ -307,6 +320,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     l_run[rt] = l;
+    m_run[rt] *= a.scale_log2;  // from here on in units of log 2, as the merges take it
   }
   if (NW > 1) {
     // every wavefront leaves (max, sum, weighted values) of its rows; wavefront 0 adds them in order
@@ -333,7 +347,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
       for (int w = 0; w < NW; ++w) {
         const float* row = wg_part + ((size_t)w * 16 * RT + rt * 16 + r) * ROW;
         const float mw = row[0];
-        const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - m);
+        const float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
         l += f * row[1];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[rt][dt] += f * *(const f32x4_t*)(row + 4 + dt * 16 + q * 4);
@@ -373,8 +387,9 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
 }
 
 // Adds the partial results of split tiles, always in split order.  One wavefront
-// per (tile, kv head, row); lane i first takes the statistics of split i, then
-// every lane sums one (or more) of the row's d outputs over the splits.
+// per (tile, kv head, row): lane i takes the statistics of split i (of splits i, i + 64, ..),
+// then every lane sums one (or more) of the row's d outputs over the splits, with the
+// weights handed from lane to lane.
 __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D, int row_tiles) {
   const int tile = blockIdx.x, kvh = blockIdx.y;
   const int lane = threadIdx.x & 63;
@@ -383,32 +398,48 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D,
   const TileRange t = tile_range(a, tile, row_tiles);
   const int nsp = t.s_last - t.s_first + 1;
   if (nsp == 1) return;
-  const int base = t.row0[row >> 4];
+  const int base = row < 16 ? t.row0[0] : t.row0[1];
   const int flat = base + (row & 15);
   if (base < 0 || flat >= t.n_rows) return;
   const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
   const float* ml = a.part_ml + (item0 * rows_per_tile + row) * 2;  // split sp is sp * rows_per_tile * 2 further
   const size_t ml_step = (size_t)rows_per_tile * 2;
+  const float* po = a.part_o + (item0 * rows_per_tile + row) * D;
+  const size_t po_step = (size_t)rows_per_tile * D;
+  const int tok = flat / a.group, g = flat - tok * a.group;
+  bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
   float m = -INFINITY;
   for (int sp = lane; sp < nsp; sp += 64) m = fmaxf(m, ml[sp * ml_step]);
   m = wave_max(m);
+  if (nsp <= 64) {
+    float w = 0.f, l = 0.f;
+    if (lane < nsp) {
+      const float ms = ml[lane * ml_step];
+      w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m);
+      l = w * ml[lane * ml_step + 1];
+    }
+    const float inv = 1.0f / wave_sum(l);
+    for (int d0 = 0; d0 < D; d0 += 64) {  // every lane stays in the loop: the weights come from all of them
+      const int d = min(d0 + lane, D - 1);
+      float o = 0.f;
+#pragma unroll 8
+      for (int sp = 0; sp < nsp; ++sp) o += __shfl(w, sp, 64) * po[sp * po_step + d];
+      if (d0 + lane < D) op[d] = __float2bfloat16(o * inv);
+    }
+    return;
+  }
   float l = 0.f;
   for (int sp = lane; sp < nsp; sp += 64) {
     const float ms = ml[sp * ml_step];
-    l += (ms == -INFINITY ? 0.f : exp2f(ms - m)) * ml[sp * ml_step + 1];
+    l += (ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m)) * ml[sp * ml_step + 1];
   }
-  l = wave_sum(l);
-  const float inv = 1.0f / l;
-  const int tok = flat / a.group, g = flat - tok * a.group;
-  bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
-  const float* po = a.part_o + (item0 * rows_per_tile + row) * D;
-  const size_t po_step = (size_t)rows_per_tile * D;
+  const float inv = 1.0f / wave_sum(l);
   for (int d = lane; d < D; d += 64) {
     float o = 0.f;
 #pragma unroll 8
     for (int sp = 0; sp < nsp; ++sp) {
       const float ms = ml[sp * ml_step];
-      const float w = ms == -INFINITY ? 0.f : exp2f(ms - m);
+      const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m);
       o += w * po[sp * po_step + d];
     }
     op[d] = __float2bfloat16(o * inv);
@@ -460,6 +491,7 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
   TK_REQUIRE(n_tiles >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_mfma: bad sizes tiles=%d nq=%d nkv=%d", n_tiles, nq, nkv);
   TK_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attention_mfma: head size %d is not a multiple of 16 up to 128", d);
   TK_REQUIRE(P >= 4 && (P & (P - 1)) == 0, "attention_mfma: page size %d is not a power of two from 4", P);
+  TK_REQUIRE(scale > 0.f, "attention_mfma: the scale must be positive");
   TK_REQUIRE(row_tiles == 1 || row_tiles == 2, "attention_mfma: row_tiles %d outside 1..2", row_tiles);
   TK_REQUIRE(row_tiles == 2 || !tile_row1, "attention_mfma: second row tiles given with one row tile a wavefront");
   TK_REQUIRE(split > 0 && split % 32 == 0, "attention_mfma: split %d is not a multiple of 32", split);

@@ -46,6 +46,11 @@ HIPCC_FLAGS = [
 ]
 
 
+# The attention kernel rescales its accumulators between matrix products: they stay in
+# ordinary vector registers instead of moving to and from the accumulation registers.
+SOURCE_FLAGS = {"attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 class BuildError(RuntimeError):
     pass
 
@@ -64,6 +69,7 @@ def _hipcc() -> str:
 def _digest(group: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(repr(sorted(SOURCE_FLAGS.items())).encode())
     for p in sorted(CSRC.glob("*.h")) + sources(group):
         h.update(p.name.encode())
         h.update(p.read_bytes())
@@ -114,7 +120,7 @@ def _say(msg: str) -> None:
 
 def _compile_one(hipcc: str, src: Path, obj: Path) -> tuple[Path, float]:
     t0 = time.time()
-    cmd = [hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc, *HIPCC_FLAGS, *SOURCE_FLAGS.get(src.name, []), "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise BuildError(f"hipcc failed on {src.name}:\n{proc.stderr[-4000:]}")
