@@ -58,6 +58,7 @@ def parse() -> argparse.Namespace:
     p.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has (recorded in config)")
     p.add_argument("--points", default="1,64", help="other decode batch sizes to measure, comma separated ('' for none)")
     p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--prefill-only", action="store_true", help="time only the prefill (for profiles); prints its record alone")
     p.add_argument("--eager", action="store_true", help="no HIP graphs")
     return p.parse_args()
 
@@ -193,6 +194,13 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
 
+    if args.prefill_only:
+        pdt = time_prefill(runner, PREFILL_TOKENS)
+        say(f"prefill of {PREFILL_TOKENS} tokens: {pdt * 1e3:.2f} ms")
+        flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], PREFILL_TOKENS)
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pdt, 1), "tokens": PREFILL_TOKENS, "ms": round(pdt * 1e3, 3),
+                                      "frac": round(flops / pdt / 1e12 / PEAK_TFLOPS[key], 4)}}))
+        return 0
     dt, mean_ctx = time_decode(runner, args, args.batch, args.context, args.steps, args.warmup)
     value = args.batch / dt
     nbytes = decode_bytes(runner.model, cfgd, args.batch, mean_ctx, elem)

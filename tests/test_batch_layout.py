@@ -40,3 +40,41 @@ def test_bad_entries_are_refused():
         layout([ok, ok], 100, 1)
     with pytest.raises(ValueError, match="no tokens"):
         layout([PlannedEntry("a", [], [], 0, 0, [[0]])], 100, 1)
+
+
+def test_attention_tiles_cover_every_row_tile_once():
+    """Row tiles of 16 rows: one a wavefront, two neighbours, or an early one paired
+    with a late one (a prompt under a causal mask); each exactly once."""
+    from tokasaurus_amd.kernels.ops import attention_tiles
+
+    q_lens, group = [1, 37, 0, 300, 4], 4
+    for row_tiles, pair in ((1, False), (2, False), (2, True)):
+        req, row0, row1 = attention_tiles(q_lens, group, row_tiles, pair=pair)
+        assert (row1 is not None) == pair
+        seen = []
+        for i, (r, a) in enumerate(zip(req, row0)):
+            seen.append((r, a))
+            b = row1[i] if pair else (a + 16 if row_tiles == 2 else -1)
+            if b >= 0 and b < q_lens[r] * group:
+                seen.append((r, b))
+        want = [(r, 16 * i) for r, n in enumerate(q_lens) for i in range(-(-n * group // 16))]
+        assert sorted(seen) == want, (row_tiles, pair)
+    # pairs: the keys the two tiles walk add up to about the same for every wavefront
+    req, row0, row1 = attention_tiles([300], group, 2, pair=True)
+    sums = [a + b for a, b in zip(row0, row1) if b >= 0]
+    assert len(set(sums)) == 1
+    # a subset of the requests
+    req, row0, _ = attention_tiles(q_lens, group, 1, requests=[0, 4])
+    assert req == [0, 4] and row0 == [0, 0]
+
+
+def test_attention_split_is_a_multiple_of_what_the_wavefronts_cut():
+    from tokasaurus_amd.kernels.ops import attention_max_waves, attention_split
+
+    for head_dim in (64, 128):
+        for tiles in (1, 3, 8, 64, 500):
+            for kv in (1, 100, 1024, 8192, 131072):
+                split, waves = attention_split(kv, tiles, 8, head_dim)
+                assert split % (32 * waves) == 0 and 1 <= waves <= attention_max_waves(head_dim, 1)
+                assert -(-kv // split) <= 16, "more splits than the merge is meant for"
+    assert attention_split(8192, 8, 8) == (2048, 8) and attention_split(8192, 64, 8) == (8192, 16)

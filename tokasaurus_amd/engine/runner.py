@@ -70,11 +70,12 @@ class RecordedDecodeStep:
     All of the step's integers and the sampler's numbers live in one device buffer
     that is refilled by a single copy from pinned host memory before each replay.
     Padding rows belong to no request: they read and write the null page and the
-    extra slot.  The step's attention is planned for the longest context a request
-    may have, so the same recording serves every length.
+    extra slot.  The step is planned for contexts up to ``kv_bound`` (a power of two,
+    at most the longest context a request may have), so one recording serves every
+    length up to there; an eager step plans for the same bound and so gives the same bits.
     """
 
-    def __init__(self, runner: "ModelRunner", size: int):
+    def __init__(self, runner: "ModelRunner", size: int, kv_bound: int):
         # no reference to the runner is kept: a runner and its recorded steps must not form a
         # cycle, or they would be freed by the cyclic collector at a time of its choosing,
         # possibly while another step is being recorded, when memory must not be released
@@ -108,10 +109,11 @@ class RecordedDecodeStep:
             num_tokens=B, num_requests=B, dtype=model.dtype, device=device,
             token_ids=view("token_ids"), positions=view("positions"), token_req=view("token_req"),
             q_start=view("q_start"), kv_len=view("kv_len"), slots=view("slots"),
-            host_q_start=list(range(B + 1)), host_kv_len=[runner.max_tokens_per_request] * B, host_slots=[self.null_slot] * B,
-            last_token=storage.last_token, max_q_len=1, max_kv_len=runner.max_tokens_per_request,
+            host_q_start=list(range(B + 1)), host_kv_len=[kv_bound] * B, host_slots=[self.null_slot] * B,
+            last_token=storage.last_token, max_q_len=1, max_kv_len=kv_bound,
         )
         self.ctx.extras["static"] = True  # parts keep what they plan: the step is replayed
+        self.ctx.extras["kv_bound"] = kv_bound
         self.ctx.extras["num_portions"] = 0
         tables = [view(f"table{g}").view(B, w) for g, w in enumerate(widths)]
         self.caches = runner.cache_views(tables)
@@ -133,7 +135,9 @@ class RecordedDecodeStep:
             torch.cuda.current_stream().wait_stream(stream)
             torch.cuda.synchronize()
             self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph):
+            # recorded steps run one at a time and their results are read before the next step:
+            # they share one pool of memory
+            with torch.cuda.graph(self.graph, pool=runner.graph_pool):
                 self.logits, self.ids, self.logprobs = self._forward()
             torch.cuda.synchronize()
         finally:
@@ -226,7 +230,8 @@ class ModelRunner:
         if use_graphs and max_slots < graph_max_size and max_slots not in self.graph_sizes:
             self.graph_sizes.append(max_slots)
             self.graph_sizes.sort()
-        self.recorded: dict[int, RecordedDecodeStep] = {}
+        self.recorded: dict[tuple[int, int], RecordedDecodeStep] = {}  # by (rows, context bound)
+        self.graph_pool = torch.cuda.graph_pool_handle() if use_graphs else None
         self.storage = CacheStorage(
             self.groups,
             [num_pages] * len(self.groups),
@@ -314,9 +319,20 @@ class ModelRunner:
         if any(e.q_len != 1 or e.want != [0] for e in planned):
             return None
         size = next(b for b in self.graph_sizes if b >= len(planned))
-        if size not in self.recorded:
-            self.recorded[size] = RecordedDecodeStep(self, size)
-        return self.recorded[size]
+        key = (size, self.kv_bound(max(e.start + e.q_len for e in planned)))
+        if key not in self.recorded:
+            self.recorded[key] = RecordedDecodeStep(self, *key)
+        return self.recorded[key]
+
+    def kv_bound(self, max_kv_len: int) -> int:
+        """The context length a step is planned for: the power of two from 1024 that
+        holds the step's longest request, at most the longest a request may get.  Parts
+        choose their launches from it and not from the batch's own lengths, so a recorded
+        step and an eager one cut their work alike."""
+        bound = 1024
+        while bound < max_kv_len:
+            bound *= 2
+        return min(bound, self.max_tokens_per_request)
 
     def run(self, entries: list[StepEntry], sampling: Sampling | None = None, write_slots: bool | None = None) -> StepOutput:
         """Run one batch.  Logits [wanted, vocab] float32 come in the order of the
@@ -330,6 +346,7 @@ class ModelRunner:
         else:
             hb = layout(planned, self.model.spec.vocab_size, len(self.groups))
             ctx, want_rows, tables = to_device(hb, self.model.dtype, self.model.device, self.storage.last_token)
+            ctx.extras["kv_bound"] = self.kv_bound(ctx.max_kv_len)
             logits = self.model.forward(ctx, self.cache_views(tables), self.storage.states, want_rows)
             out = StepOutput(logits)
             if sampling is not None and logits.shape[0] > 0:

@@ -355,18 +355,23 @@ def attention_max_waves(head_dim: int, row_tiles: int) -> int:
 
 
 def attention_split(max_kv_len: int, n_tiles: int, nkv: int, head_dim: int = 64) -> tuple[int, int]:
-    """(keys per split, wavefronts per workgroup) for tiles of one row tile.  With few
-    tiles (decode) the keys are cut so that about four thousand wavefronts share the
-    work, each with 64 to 512 keys, 4 to 16 of them a workgroup (measured best on an
-    MI355X at 8192 keys: 64 keys x 4 at batch 1, 128 x 8 at batch 8, 512 x 16 at batch
-    64); with thousands of tiles nothing is split and a workgroup is one wavefront."""
+    """(keys per split, wavefronts per workgroup) for tiles of one row tile (decode).
+    The keys of a tile are cut into at most 16 splits so that there are about 256
+    workgroups (one a compute unit); the wavefronts of a workgroup, which adds their
+    results itself, take 64 to 512 keys each, about two thousand wavefronts in all.
+    Measured best on an MI355X at 8192 keys, with the cache read from memory:
+    64 keys x 8 wavefronts x 16 splits at batch 1, 256 x 8 x 4 at batch 8,
+    512 x 16 x 1 at batch 64."""
     base = max(n_tiles * nkv, 1)
-    whole = -(-max(max_kv_len, 1) // 128) * 128
-    if base >= 2048:
-        return whole, 1
-    sub = min(512, max(64, -(-(max_kv_len * base // 4096) // 32) * 32))
-    waves = min(4 if base <= 16 else (8 if base <= 128 else 16), attention_max_waves(head_dim, 1))
-    return sub * waves, waves
+    kv = max(max_kv_len, 1)
+    splits = max(1, min(16, -(-256 // base)))
+    raw = -(-kv // splits)
+    per_wave = min(512, max(64, kv * base // 2048))
+    waves = 1
+    while waves * 2 <= min(attention_max_waves(head_dim, 1), raw // per_wave):
+        waves *= 2
+    step = 32 * waves
+    return -(-raw // step) * step, waves
 
 
 class AttentionScratch:
@@ -417,12 +422,14 @@ def paged_attention_mfma(
     out: torch.Tensor | None = None,
     scratch: "AttentionScratch | None" = None,
     tile_row1: torch.Tensor | None = None,
+    longest: int | None = None,
 ) -> torch.Tensor:
     """Attention of every token of the batch over its request's pages on the
     matrix cores (bfloat16).  ``q`` is 2-d and its first nq*d columns are the
     query heads; request r owns tokens q_start[r]..q_start[r+1]-1, the last of
     them at position kv_len[r]-1.  ``max_kv_len`` bounds kv_len (it sizes the
-    grid and the scratch, so it may be larger than any request's).  The tiles
+    grid and the scratch, so it may be larger than any request's; ``longest``, if
+    given, is the length of the longest request, which the block table must cover).  The tiles
     (see ``attention_tiles``) may cover some of the requests only; rows of ``out``
     that no tile covers are left as they are."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0)
@@ -436,8 +443,9 @@ def paged_attention_mfma(
     requests = kv_len.numel()
     _need(q_start.numel() == requests + 1 and block_table.shape[0] >= requests,
           "attention_mfma: q_start, kv_len and block_table disagree on the number of requests")
-    _need(block_table.shape[1] * page_size >= max_kv_len or requests == 0,
+    _need(block_table.shape[1] * page_size >= (max_kv_len if longest is None else longest) or requests == 0,
           "attention_mfma: block table narrower than the longest request")
+    _need(longest is None or longest <= max_kv_len, "attention_mfma: the longest request exceeds max_kv_len")
     n_tiles = tile_req.numel()
     _need(tile_row0.numel() == n_tiles, "attention_mfma: tile lists differ in length")
     if tile_row1 is not None:

@@ -63,14 +63,16 @@ def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int) -> Att
         small = [r for r, n in enumerate(q_lens) if 0 < n * group <= 16]
         large = [r for r, n in enumerate(q_lens) if n * group > 16]
         static = bool(ctx.extras.get("static"))
+        # launches are chosen for the bound the step was planned for, not for the lengths in it
+        bound = max(int(ctx.extras.get("kv_bound", 0)), ctx.max_kv_len)
         lists: list[tuple[list[int], list[int], list[int] | None, int, int, int]] = []
         if small:
             req, row0, _ = ops.attention_tiles(q_lens, group, 1, small)
-            split, waves = ops.attention_split(ctx.max_kv_len, len(req), nkv, head_dim)
+            split, waves = ops.attention_split(bound, len(req), nkv, head_dim)
             lists.append((req, row0, None, 1, split, waves))
         if large:
             req, row0, row1 = ops.attention_tiles(q_lens, group, 2, large, pair=True)
-            whole = -(-max(ctx.max_kv_len, 1) // 128) * 128
+            whole = -(-max(bound, 1) // 128) * 128
             lists.append((req, row0, row1, 2, whole, 1))
         # one upload for all the tile lists of the step
         flat = [x for req, row0, row1, *_ in lists for x in (req + row0 + (row1 or []))]
@@ -83,7 +85,7 @@ def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int) -> Att
             at += (3 if row1 is not None else 2) * n
             launches.append(AttentionLaunch(t_req, t_row0, t_row1, row_tiles, split, waves,
                                             ops.AttentionScratch(ctx.device) if static else None))
-        plan = AttentionPlan(launches, ctx.max_kv_len)
+        plan = AttentionPlan(launches, bound)
         ctx.extras[key] = plan
     return plan
 
@@ -169,7 +171,7 @@ class PagedAttention(Mixer):
                     q, cache.keys, cache.values, cache.block_table, ctx.q_start, ctx.kv_len,
                     launch.tile_req, launch.tile_row0, launch.row_tiles, nq, nkv, d, cache.page_size,
                     plan.max_kv_len, launch.split, window=self.window, scale=self.scale, waves=launch.waves,
-                    out=attn, scratch=launch.scratch, tile_row1=launch.tile_row1,
+                    out=attn, scratch=launch.scratch, tile_row1=launch.tile_row1, longest=ctx.max_kv_len,
                 )
         else:
             # the true 32-bit path, and shapes the matrix-core kernel does not take
