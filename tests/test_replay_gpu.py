@@ -22,7 +22,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": [5, 17, 33, 97], "B": [1, 9, 70, 130], "C": [40, 150]}
+LENGTHS = {"A": [5, 17, 33, 97], "B": [1, 9, 70, 130], "C": [40, 150], "D": [3, 66, 131]}
 
 
 def requests_for(name):
@@ -36,7 +36,7 @@ def runner_for(folders, name, dtype, tokens=512):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_each_request_alone_and_whole(folders, name, dtype):
     reqs = requests_for(name)
     ref = plain_rows(folders[name], reqs)
@@ -49,7 +49,7 @@ def test_each_request_alone_and_whole(folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_last_32_tokens_one_by_one(folders, name, dtype):
     reqs = {k: v for k, v in requests_for(name).items() if len(v) > 32}
     ref = plain_rows(folders[name], reqs)
@@ -61,7 +61,7 @@ def test_last_32_tokens_one_by_one(folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_portions_of_changing_size(folders, name, dtype):
     reqs = requests_for(name)
     ref = plain_rows(folders[name], reqs)
@@ -101,10 +101,11 @@ def mixed_trace(reqs: dict[str, list[int]], seed: int, max_live: int = 4):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_mixed_batches_with_pages_used_again(folders, name, dtype):
     cfg, page = TINY[name]
-    lengths = {"A": [33, 50, 21, 60, 44, 9, 38], "B": [70, 9, 130, 1, 55, 64, 90], "C": [80, 150, 33, 100, 17]}[name]
+    lengths = {"A": [33, 50, 21, 60, 44, 9, 38], "B": [70, 9, 130, 1, 55, 64, 90], "C": [80, 150, 33, 100, 17],
+               "D": [66, 131, 20, 97, 40, 70]}[name]
     reqs = {f"m{i}": random_tokens(n, cfg["vocab_size"], 500 + i) for i, n in enumerate(lengths)}
     ref = plain_rows(folders[name], reqs)
     # room for the four longest at once, each rounded up to 64 tokens: far fewer pages than the sum

@@ -85,7 +85,27 @@ CONFIG_C = {
 }
 PAGE_C = 16
 
-TINY = {"A": (CONFIG_A, PAGE_A), "B": (CONFIG_B, PAGE_B), "C": (CONFIG_C, PAGE_C)}
+# awkward sizes: no grouping (as many kv heads as heads), an intermediate size that is no
+# multiple of 8 (the bfloat16 matrix-core products cannot take it: the plain kernel does),
+# an odd vocabulary, one layer, a large eps, pages of 32
+CONFIG_D = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "num_hidden_layers": 1,
+    "hidden_size": 80,
+    "num_attention_heads": 5,
+    "num_key_value_heads": 5,
+    "intermediate_size": 172,
+    "vocab_size": 333,
+    "rope_theta": 1234.5,
+    "rope_scaling": None,
+    "rms_norm_eps": 1e-3,
+    "tie_word_embeddings": False,
+    "max_position_embeddings": 300,
+}
+PAGE_D = 32
+
+TINY = {"A": (CONFIG_A, PAGE_A), "B": (CONFIG_B, PAGE_B), "C": (CONFIG_C, PAGE_C), "D": (CONFIG_D, PAGE_D)}
 
 
 def make_folder(folder: Path, config: dict, seed: int, sharp: bool = True) -> Path:

@@ -52,12 +52,6 @@ class Linear:
         return [TensorSpec(n, (o, self.in_features), MATRIX) for n, o in zip(self.names, self.out_features)]
 
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
-        if placer.dtype == torch.bfloat16 and self.in_features % 8:
-            raise ValueError(
-                f"{self.names[0]}: the bfloat16 kernels need an inner size that is a multiple of 8, "
-                f"got {self.in_features}; run this model with dtype=float32"
-            )
-
         def make() -> torch.Tensor:
             parts = [tensors[n] for n in self.names]
             w = parts[0] if len(parts) == 1 else torch.cat(parts, dim=0)
@@ -65,8 +59,12 @@ class Linear:
 
         self.weight = placer.place(("row_major", *self.names), make)
 
+    def _aligned(self) -> bool:
+        # the bfloat16 matrix-core kernels read 8 inputs (16 bytes) at a time
+        return self.weight.shape[1] % 8 == 0
+
     def _fast(self, m: int) -> bool:
-        return self.weight.dtype == torch.bfloat16 and 0 < m <= ops.SKINNY_MAX_ROWS
+        return self.weight.dtype == torch.bfloat16 and 0 < m <= ops.SKINNY_MAX_ROWS and self._aligned()
 
     def __call__(
         self,
@@ -93,7 +91,7 @@ class Linear:
             else:
                 x = x.materialize()
         m = x.shape[0]
-        if w.dtype == torch.bfloat16 and m > 0:
+        if w.dtype == torch.bfloat16 and m > 0 and (m > ops.SKINNY_MAX_ROWS or self._aligned()):
             if m <= ops.SKINNY_MAX_ROWS:
                 return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu,
                                             prenorm=prenorm, norm_eps=eps)
@@ -104,6 +102,7 @@ class Linear:
             if swiglu:
                 return ops.swiglu(prod)
             return prod.float() if out_f32 else prod
+        # the 32-bit path, and few bfloat16 rows of a width the matrix-core kernel does not take
         out = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)
         return ops.swiglu(out) if swiglu else out
 
