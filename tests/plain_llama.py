@@ -193,13 +193,14 @@ def lm_head(x: torch.Tensor, w: dict[str, torch.Tensor], cfg: dict) -> torch.Ten
 
 
 def load_folder(folder: str | Path) -> tuple[dict, dict[str, torch.Tensor]]:
-    """config.json as a dict and every tensor of model.safetensors in 32-bit."""
+    """config.json as a dict and every tensor of model.safetensors in 32-bit (tables of integers as they are)."""
     folder = Path(folder)
     cfg = json.loads((folder / "config.json").read_text())
     weights = {}
     with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
         for name in f.keys():
-            weights[name] = f.get_tensor(name).to(torch.float32)
+            t = f.get_tensor(name)
+            weights[name] = t.to(torch.float32) if t.is_floating_point() else t
     return cfg, weights
 
 

@@ -238,6 +238,40 @@ def test_a_mixer_with_state_of_its_own(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_feed_forward_with_routing_and_another_position_encoding(tmp_path, dtype):
+    """Layers 0 and 2 route each token to one of four toy experts through an integer
+    table of the checkpoint; every layer rotates by the toy's own angles.  Requests are
+    drawn so that no routing decision is close: a token near a tie may go to another
+    expert in bfloat16, which is no fault of the engine's."""
+    toy_parts.register()
+    config = dict(CONFIG_A, model_type="toy_mixture", num_hidden_layers=3, toy_routed_layers=[0, 2], toy_num_experts=4,
+                  toy_expert_size=40, toy_angle_rate=0.37)
+    folder = write_random_model(tmp_path / "mixture", config, seed=9)
+    sharpen(folder, {"router.weight": 40.0, "in.weight": 6.0, "out.weight": 6.0, "q_proj.weight": math.sqrt(3.0 / 64) / 0.02,
+                     "k_proj.weight": math.sqrt(3.0 / 64) / 0.02})
+    cfg, w = plain_llama.load_folder(folder)
+    assert w["model.layers.0.moe.rename"].dtype == torch.int32
+    reqs, ref, seed = {}, {}, 0
+    for n in (14, 30, 7, 22, 3):
+        while True:
+            seed += 1
+            toks = random_tokens(n, cfg["vocab_size"], 1000 + seed)
+            logits, margin = toy_parts.plain_toy_mixture_logits(cfg, w, toks)
+            if margin > 0.04:  # in units of the spread of the router logits; bfloat16 moves them by a few thousandths
+                break
+            assert seed < 3000, "no request without a close routing decision found"
+        reqs[f"x{n}"], ref[f"x{n}"] = toks, logits
+    # the experts and the angles matter: other choices give other logits
+    other = dict(w)
+    other["model.layers.0.moe.rename"] = w["model.layers.0.moe.rename"] + 1
+    assert (toy_parts.plain_toy_mixture_logits(cfg, other, reqs["x30"])[0] - ref["x30"]).abs().max() > 0.05
+    assert (toy_parts.plain_toy_mixture_logits(dict(cfg, toy_angle_rate=0.2), w, reqs["x30"])[0] - ref["x30"]).abs().max() > 0.05
+    runner = ModelRunner.from_folder(folder, dtype, page_size=4, num_pages=64, max_slots=4)
+    all_cuttings(runner, reqs, ref, TOL[dtype])
+    assert runner.recorded, "decode steps of the toy model were not recorded"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_run_order_as_data_and_a_shared_cache(tmp_path, dtype):
     """Layer 0 runs twice (each use with a cache of its own) and the last entry
     reads the cache of the second instead of keeping one."""

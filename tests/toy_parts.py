@@ -1,8 +1,10 @@
 """Parts and architectures that exist only in the tests.  They are registered
 through the framework's public registries, without a change to its files, and
 show what the interfaces carry: a mixer with per-request state of its own, a
-run order that names a layer twice and lets an entry read another entry's cache,
-and layers with a sliding window (a cache group of their own).  None of them is
+feed-forward that routes tokens to experts through a table of integers, a position
+encoding with angles of its own, a run order that names a layer twice and lets an
+entry read another entry's cache, and layers with a sliding window (a cache group
+of their own).  None of them is
 a model of anyone's; the plain references sit beside them.
 """
 
@@ -18,7 +20,19 @@ from tokasaurus_amd.config.model_config import LlamaConfig
 from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.models import Architecture, ModelSpec, RunEntry, register_architecture
 from tokasaurus_amd.models.llama import llama_spec
-from tokasaurus_amd.parts.base import MIXERS, NORM_WEIGHT, Mixer, PartSpec, StateNeed, TensorSpec
+from tokasaurus_amd.parts.base import (
+    FEED_FORWARDS,
+    INT_TABLE,
+    MIXERS,
+    NORM_WEIGHT,
+    POSITION_ENCODINGS,
+    FeedForward,
+    Mixer,
+    PartSpec,
+    PositionEncoding,
+    StateNeed,
+    TensorSpec,
+)
 from tokasaurus_amd.parts.linear import Linear
 
 # --------------------------------------------------------------------------
@@ -129,6 +143,141 @@ def plain_toy_recurrent_logits(cfg: dict, w: dict, token_ids: list[int]) -> torc
 
 
 # --------------------------------------------------------------------------
+# a feed-forward with routing, and a position encoding with other angles
+# --------------------------------------------------------------------------
+
+
+@FEED_FORWARDS.register("toy_routed", replace=True)
+class ToyRouted(FeedForward):
+    """A token goes to ONE of a few small experts (two products with a ReLU between):
+    the one whose router logit (32-bit) is largest, renamed through a table of
+    integers from the checkpoint; its output is weighted with the softmax
+    probability of that logit.  Every expert runs on every token and a mask picks:
+    a toy has no need for a gather, and the step stays free of host decisions."""
+
+    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, names: dict[str, str]):
+        self.num_experts = num_experts
+        self.router = Linear(hidden_size, [names["router"]], [num_experts])
+        self.w_in = [Linear(hidden_size, [names["in"].format(e)], [expert_size]) for e in range(num_experts)]
+        self.w_out = [Linear(expert_size, [names["out"].format(e)], [hidden_size]) for e in range(num_experts)]
+        self.rename_name = names["rename"]
+        self.rename: torch.Tensor | None = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        specs = self.router.tensor_specs() + [TensorSpec(self.rename_name, (self.num_experts,), INT_TABLE)]
+        for lin in self.w_in + self.w_out:
+            specs += lin.tensor_specs()
+        return specs
+
+    def load(self, tensors, placer) -> None:
+        for lin in [self.router] + self.w_in + self.w_out:
+            lin.load(tensors, placer)
+        assert tensors[self.rename_name].dtype == torch.int32, "an integer table must arrive as int32"
+        self.rename = placer.place(("table", self.rename_name), lambda: tensors[self.rename_name].to(placer.device))
+
+    def forward(self, h, residual):
+        logits = ops.gemm_generic(h, self.router.weight, out_f32=True)  # [N, E] 32-bit
+        top = logits.argmax(-1)
+        weight = torch.softmax(logits, -1).gather(-1, top[:, None])
+        expert = self.rename[top].long() % self.num_experts
+        y = torch.zeros((h.shape[0], residual.shape[1]), dtype=torch.float32, device=h.device)
+        for e in range(self.num_experts):
+            out = self.w_out[e](torch.relu(self.w_in[e](h)))
+            y = torch.where((expert == e)[:, None], out.float(), y)
+        return ops.add((weight * y).to(h.dtype), residual.contiguous())
+
+
+def plain_routed(h: torch.Tensor, w: dict, prefix: str, num_experts: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """The toy feed-forward on [T, H]; also each token's margin: the gap between its two
+    largest router logits relative to their spread (a small one may fall either way
+    in reduced precision)."""
+    logits = h @ w[f"{prefix}.moe.router.weight"].T
+    top = logits.argmax(-1)
+    weight = torch.softmax(logits, -1).gather(-1, top[:, None])
+    expert = w[f"{prefix}.moe.rename"].long()[top] % num_experts
+    out = torch.zeros_like(h)
+    for t in range(h.shape[0]):
+        e = int(expert[t])
+        out[t] = w[f"{prefix}.moe.experts.{e}.out.weight"] @ torch.relu(w[f"{prefix}.moe.experts.{e}.in.weight"] @ h[t])
+    two = logits.topk(2, -1).values
+    margin = (two[:, 0] - two[:, 1]) / logits.std(-1).clamp_min(1e-9)
+    return weight * out, margin
+
+
+@POSITION_ENCODINGS.register("toy_angles", replace=True)
+class ToyAngles(PositionEncoding):
+    """Rotation by pos * rate / (j + 1) for pair j: tables of its own making, in the form the
+    attention part takes them (cos and sin [positions, d/2], 32-bit, on the device)."""
+
+    def __init__(self, head_dim: int, rate: float, max_positions: int):
+        self.head_dim, self.rate, self.max_positions = head_dim, float(rate), int(max_positions)
+        self.cos: torch.Tensor | None = None
+        self.sin: torch.Tensor | None = None
+
+    def prepare(self, device: torch.device) -> None:
+        if self.cos is None:
+            angles = toy_angles(self.head_dim, self.rate, torch.arange(self.max_positions)).to(device)
+            self.cos, self.sin = torch.cos(angles).contiguous(), torch.sin(angles).contiguous()
+
+
+def toy_angles(head_dim: int, rate: float, positions: torch.Tensor) -> torch.Tensor:
+    return positions[:, None].to(torch.float32) * (rate / torch.arange(1, head_dim // 2 + 1, dtype=torch.float32))[None, :]
+
+
+@dataclass(frozen=True)
+class MixtureConfig:
+    llama: LlamaConfig
+    routed_layers: tuple[int, ...]
+    num_experts: int
+    expert_size: int
+    angle_rate: float
+
+    @staticmethod
+    def from_dict(d: dict[str, Any]) -> "MixtureConfig":
+        return MixtureConfig(LlamaConfig.from_dict(d), tuple(d["toy_routed_layers"]), int(d["toy_num_experts"]),
+                             int(d["toy_expert_size"]), float(d["toy_angle_rate"]))
+
+
+def toy_mixture_spec(cfg: MixtureConfig) -> ModelSpec:
+    base = llama_spec(cfg.llama)
+    position = PartSpec("toy_angles", {"head_dim": cfg.llama.head_dim, "rate": cfg.angle_rate,
+                                       "max_positions": cfg.llama.max_position_embeddings})
+    layers = []
+    for i, layer in enumerate(base.layers):
+        params = dict(layer.params)
+        mixer = params["mixer"]
+        params["mixer"] = PartSpec(mixer.kind, {**mixer.params, "position": position})
+        if i in cfg.routed_layers:
+            p = f"model.layers.{i}.moe"
+            params["feed_forward"] = PartSpec("toy_routed", {
+                "hidden_size": cfg.llama.hidden_size, "expert_size": cfg.expert_size, "num_experts": cfg.num_experts,
+                "names": {"router": f"{p}.router.weight", "rename": f"{p}.rename",
+                          "in": p + ".experts.{}.in.weight", "out": p + ".experts.{}.out.weight"}})
+        layers.append(PartSpec(layer.kind, params))
+    return ModelSpec(**{**base.__dict__, "layers": tuple(layers)})
+
+
+def plain_toy_mixture_logits(cfg: dict, w: dict, token_ids: list[int]) -> tuple[torch.Tensor, float]:
+    """Logits [T, V] and the smallest routing margin of the sequence."""
+    d = cfg["hidden_size"] // cfg["num_attention_heads"]
+    x = w["model.embed_tokens.weight"][torch.tensor(token_ids)]
+    angles = toy_angles(d, float(cfg["toy_angle_rate"]), torch.arange(len(token_ids)))
+    cos, sin = torch.cos(torch.cat([angles, angles], -1)), torch.sin(torch.cat([angles, angles], -1))
+    smallest = float("inf")
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}"
+        x = plain_llama.attention_block(x, w, p, cfg, cos, sin)
+        if i in cfg["toy_routed_layers"]:
+            h = plain_llama.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], cfg["rms_norm_eps"])
+            y, margin = plain_routed(h, w, p, cfg["toy_num_experts"])
+            x = x + y
+            smallest = min(smallest, float(margin.min()))
+        else:
+            x = plain_llama.swiglu_block(x, w, p, cfg)
+    return plain_llama.lm_head(x, w, cfg), smallest
+
+
+# --------------------------------------------------------------------------
 # Llama's parts in another arrangement: a run order as data, windows per layer
 # --------------------------------------------------------------------------
 
@@ -167,3 +316,4 @@ def plain_arranged_logits(cfg: dict, w: dict, token_ids: list[int]) -> torch.Ten
 def register() -> None:
     register_architecture(Architecture("toy_recurrent", ToyConfig.from_dict, toy_recurrent_spec), replace=True)
     register_architecture(Architecture("toy_arranged", ArrangedConfig.from_dict, arranged_spec), replace=True)
+    register_architecture(Architecture("toy_mixture", MixtureConfig.from_dict, toy_mixture_spec), replace=True)
