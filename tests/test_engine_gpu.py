@@ -93,17 +93,23 @@ def test_bfloat16_generation_follows_the_plain_one(folders, name):
             ids.append(tok)
 
 
-def test_recorded_and_eager_decode_steps_agree(folders):
+@pytest.mark.parametrize("live, lengths", [(3, (30, 8, 55, 21, 40)), (40, tuple(5 + (7 * i) % 23 for i in range(44)))])
+def test_recorded_and_eager_decode_steps_agree(folders, live, lengths):
     """The same requests with and without recorded steps, several replays with eager
-    work (prompt portions of later requests) between them: the same tokens."""
+    work (prompt portions of later requests) between them: the same tokens.  With 40
+    live requests a step has more rows than the weight-streaming product takes on, so
+    the recorded steps hold library products."""
     cfg, _ = TINY["C"]
-    prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (30, 8, 55, 21, 40)]
+    prompts = [random_tokens(n, cfg["vocab_size"], 90 + n + i) for i, n in enumerate(lengths)]
     results = []
     for graphs in (True, False):
-        engine = engine_for(folders, "C", dtype="bfloat16", use_hipgraphs=graphs, max_seqs_per_forward=3, max_tokens_per_forward=32)
+        engine = engine_for(folders, "C", dtype="bfloat16", use_hipgraphs=graphs, max_seqs_per_forward=live,
+                            max_tokens_per_forward=max(32, live + 16), kv_cache_num_tokens=4096)
         done = engine.generate(prompts, SamplingParams(temperature=0.7, max_tokens=20, ignore_eos=True, seed=3))
         results.append([(c.tokens, c.logprobs) for c in done])
         assert bool(engine.runner.recorded) == graphs
+        if graphs:
+            assert max(size for size, _ in engine.runner.recorded) >= min(live, len(lengths)) - 8
     for (ta, la), (tb, lb) in zip(*results):
         assert ta == tb
         assert torch.allclose(torch.tensor(la), torch.tensor(lb), atol=1e-5)

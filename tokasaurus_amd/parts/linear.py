@@ -5,12 +5,14 @@ be stacked along the output rows into one product (q|k|v, gate|up).
 
 Which kernel runs is decided by the storage type and the number of rows:
   * float32: 32-bit multiply-adds throughout (the true 32-bit path);
-  * bfloat16, up to 128 rows (decode): the hand-written matrix-core kernel that
-    streams the weight once and fuses the epilogue; it can also fold in the norm in
-    front (``Normed`` input), leave what the norm behind it needs (``emit_norm``), and
-    rotate and append q, k and v (``rope_append``);
-  * bfloat16, more rows (prefill): the library's matrix product, as in the
-    reference (its projections are library calls), followed by the epilogue kernel.
+  * bfloat16, up to ``ops.SKINNY_ROWS`` rows (decode): the hand-written matrix-core
+    kernel that streams the weight once and fuses the epilogue; it can also fold in the
+    norm in front (``Normed`` input), leave what the norm behind it needs
+    (``emit_norm``), and rotate and append q, k and v (``rope_append``);
+  * bfloat16, more rows (large decode batches, prefill): the library's matrix product,
+    as in the reference (its projections are library calls), followed by the epilogue
+    kernel; a bfloat16 weight whose inner size is no multiple of 8 takes the plain
+    kernel for few rows.
 """
 
 from __future__ import annotations
@@ -64,7 +66,7 @@ class Linear:
         return self.weight.shape[1] % 8 == 0
 
     def _fast(self, m: int) -> bool:
-        return self.weight.dtype == torch.bfloat16 and 0 < m <= ops.SKINNY_MAX_ROWS and self._aligned()
+        return self.weight.dtype == torch.bfloat16 and 0 < m <= ops.SKINNY_ROWS and self._aligned()
 
     def __call__(
         self,
@@ -91,17 +93,17 @@ class Linear:
             else:
                 x = x.materialize()
         m = x.shape[0]
-        if w.dtype == torch.bfloat16 and m > 0 and (m > ops.SKINNY_MAX_ROWS or self._aligned()):
-            if m <= ops.SKINNY_MAX_ROWS:
+        if w.dtype == torch.bfloat16 and m > 0 and (m > ops.SKINNY_ROWS or self._aligned()):
+            if m <= ops.SKINNY_ROWS:
                 return ops.gemm_skinny_bf16(x, w, residual=residual, out_f32=out_f32, swiglu=swiglu,
                                             prenorm=prenorm, norm_eps=eps)
             # library matrix product (hipBLASLt), 32-bit accumulation
             if residual is not None:
                 return torch.addmm(residual, x, w.t())  # the residual is added in the product's epilogue
+            if out_f32:
+                return torch.mm(x, w.t(), out_dtype=torch.float32)
             prod = torch.mm(x, w.t())
-            if swiglu:
-                return ops.swiglu(prod)
-            return prod.float() if out_f32 else prod
+            return ops.swiglu(prod) if swiglu else prod
         # the 32-bit path, and few bfloat16 rows of a width the matrix-core kernel does not take
         out = ops.gemm_generic(x, w, residual=residual, out_f32=out_f32)
         return ops.swiglu(out) if swiglu else out
