@@ -311,7 +311,7 @@ def test_embed_gather_and_slot_tokens(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("hidden", [64, 96, 1000, 2048])
+@pytest.mark.parametrize("hidden", [64, 96, 1000, 2048, 37, 10240])
 def test_rmsnorm(dtype, hidden):
     import plain_llama
     from tokasaurus_amd.kernels import ops
@@ -328,6 +328,18 @@ def test_rmsnorm(dtype, hidden):
     if dtype == "bfloat16":
         got = ops.rmsnorm(x.cuda(), w.float().cuda(), 1e-5).cpu()
         assert torch.allclose(got.float(), plain_llama.rms_norm(x, w, 1e-5).float(), atol=2e-2, rtol=1e-2)
+    # the sum with a residual and its norm in one pass: the very bits of the two steps apart
+    r = torch.randn((7, hidden), generator=g).to(DT[dtype])
+    stream, normed = ops.add_rmsnorm(x.cuda(), r.cuda(), w.cuda(), 1e-5)
+    want_stream = ops.add(x.cuda(), r.cuda())
+    assert torch.equal(stream, want_stream) and torch.equal(normed, ops.rmsnorm(want_stream, w.cuda(), 1e-5))
+    assert torch.equal(stream.cpu(), (x.float() + r.float()).to(DT[dtype]))
+    # rows whose start is not 16-byte aligned take the element-wise kernel (it sums the squares in another order)
+    wide = torch.zeros((7 * hidden + 1,), dtype=DT[dtype]).cuda()
+    off = wide[1:].view(7, hidden)
+    off.copy_(x.cuda())
+    assert off.data_ptr() % 16 != 0
+    assert torch.allclose(ops.rmsnorm(off, w.cuda(), 1e-5).cpu().float(), plain_llama.rms_norm(x, w, 1e-5).float(), **tol)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -342,6 +354,9 @@ def test_swiglu_gather_add(dtype):
     tol = dict(atol=1e-6, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=2e-2)
     assert torch.allclose(got, want, **tol)
     assert float(ops.swiglu(torch.zeros((2, 8), dtype=DT[dtype]).cuda()).abs().max()) == 0.0
+    gu = torch.randn((3, 2 * 4096), generator=g).to(DT[dtype])  # a width the 16-byte kernel takes
+    want = torch.nn.functional.silu(gu[:, :4096].float()) * gu[:, 4096:].float()
+    assert torch.allclose(ops.swiglu(gu.cuda()).cpu().float(), want, **tol)
 
     src = torch.randn((9, 200), generator=g).to(DT[dtype])
     idx = torch.tensor([8, 0, 3, 3], dtype=torch.int32)

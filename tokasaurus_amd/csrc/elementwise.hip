@@ -37,28 +37,136 @@ TK_API int tk_embed_gather(int dt, const int* ids, const int* last_token, const 
 }
 
 // --------------------------------------------------------------------------
+// 16 bytes of the storage type at a time, where sizes and addresses allow it
+// --------------------------------------------------------------------------
+template <typename T>
+struct Pack {
+  static constexpr int N = 16 / sizeof(T);
+  union { uint4 raw; T v[N]; };
+  __device__ __forceinline__ void load(const T* p) { raw = *(const uint4*)p; }
+  __device__ __forceinline__ void store(T* p) const { *(uint4*)p = raw; }
+};
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// --------------------------------------------------------------------------
 // RMSNorm: statistics in 32-bit, the normalised value rounded to the storage
 // type, then multiplied by the weight and rounded again.  The weight is of the
 // storage type, or 32-bit when `w_f32` (then the product is rounded once more only).
+// With ADD the rows are first x + residual (rounded), which is also written out:
+// the residual stream and its norm in one pass.
 // --------------------------------------------------------------------------
-template <typename T>
-__global__ void rmsnorm_kernel(const T* __restrict__ x, const void* __restrict__ w, int w_f32,
+template <typename T, bool ADD>
+__global__ void rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ residual,
+                               const void* __restrict__ w, int w_f32, T* __restrict__ stream_out,
                                T* __restrict__ out, int hidden, float eps) {
   __shared__ float red[16];
   const T* row = x + (size_t)blockIdx.x * hidden;
+  const T* rrow = ADD ? residual + (size_t)blockIdx.x * hidden : nullptr;
+  T* srow = ADD ? stream_out + (size_t)blockIdx.x * hidden : nullptr;
   T* orow = out + (size_t)blockIdx.x * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = to_f32<T>(row[i]);
+    if (ADD) {
+      v = round_to<T>(v + to_f32<T>(rrow[i]));
+      srow[i] = from_f32<T>(v);
+    }
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float rstd = 1.0f / sqrtf(ss / (float)hidden + eps);
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float n = round_to<T>(to_f32<T>(row[i]) * rstd);
+    float n = round_to<T>(to_f32<T>(ADD ? srow[i] : row[i]) * rstd);  // a thread reads back what it wrote
     float wi = w_f32 ? ((const float*)w)[i] : to_f32<T>(((const T*)w)[i]);
     orow[i] = from_f32<T>(wi * n);
   }
+}
+
+// The same with 16-byte accesses; a thread keeps its first RN_HELD pieces of the row in registers.
+#define RN_HELD 4
+template <typename T, bool ADD>
+__global__ __launch_bounds__(256) void rmsnorm_packed_kernel(
+    const T* __restrict__ x, const T* __restrict__ residual, const void* __restrict__ w, int w_f32,
+    T* __restrict__ stream_out, T* __restrict__ out, int hidden, float eps) {
+  constexpr int N = Pack<T>::N;
+  __shared__ float red[16];
+  const size_t base = (size_t)blockIdx.x * hidden;
+  const int pieces = hidden / N;
+  float held[RN_HELD][N];
+  float ss = 0.f;
+  auto take = [&](int piece, float (&v)[N]) {
+    Pack<T> a;
+    a.load(x + base + (size_t)piece * N);
+    if (ADD) {
+      Pack<T> r, s;
+      r.load(residual + base + (size_t)piece * N);
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        v[j] = round_to<T>(to_f32<T>(a.v[j]) + to_f32<T>(r.v[j]));
+        s.v[j] = from_f32<T>(v[j]);
+      }
+      s.store(stream_out + base + (size_t)piece * N);
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) v[j] = to_f32<T>(a.v[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) ss += v[j] * v[j];
+  };
+#pragma unroll
+  for (int c = 0; c < RN_HELD; ++c) {
+    const int piece = threadIdx.x + c * 256;
+    if (piece < pieces) take(piece, held[c]);
+  }
+  for (int piece = threadIdx.x + RN_HELD * 256; piece < pieces; piece += 256) {
+    float v[N];
+    take(piece, v);
+  }
+  ss = block_sum(ss, red);
+  const float rstd = 1.0f / sqrtf(ss / (float)hidden + eps);
+  auto give = [&](int piece, const float (&v)[N]) {
+    Pack<T> o;
+    float wf[N];
+    if (w_f32) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) wf[j] = ((const float*)w)[(size_t)piece * N + j];
+    } else {
+      Pack<T> wp;
+      wp.load((const T*)w + (size_t)piece * N);
+#pragma unroll
+      for (int j = 0; j < N; ++j) wf[j] = to_f32<T>(wp.v[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < N; ++j) o.v[j] = from_f32<T>(wf[j] * round_to<T>(v[j] * rstd));
+    o.store(out + base + (size_t)piece * N);
+  };
+#pragma unroll
+  for (int c = 0; c < RN_HELD; ++c) {
+    const int piece = threadIdx.x + c * 256;
+    if (piece < pieces) give(piece, held[c]);
+  }
+  for (int piece = threadIdx.x + RN_HELD * 256; piece < pieces; piece += 256) {
+    Pack<T> a;
+    a.load((ADD ? stream_out : x) + base + (size_t)piece * N);  // a thread reads back what it wrote
+    float v[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) v[j] = to_f32<T>(a.v[j]);
+    give(piece, v);
+  }
+}
+
+template <typename T, bool ADD>
+static void launch_rmsnorm(const void* x, const void* residual, const void* w, int w_f32, void* stream_out,
+                           void* out, int rows, int hidden, float eps, hipStream_t stream) {
+  const bool packed = hidden % Pack<T>::N == 0 && aligned16(x) && aligned16(out) && aligned16(w) &&
+                      (!ADD || (aligned16(residual) && aligned16(stream_out)));
+  if (packed)
+    hipLaunchKernelGGL((rmsnorm_packed_kernel<T, ADD>), dim3(rows), dim3(256), 0, stream, (const T*)x,
+                       (const T*)residual, w, w_f32, (T*)stream_out, (T*)out, hidden, eps);
+  else
+    hipLaunchKernelGGL((rmsnorm_kernel<T, ADD>), dim3(rows), dim3(256), 0, stream, (const T*)x,
+                       (const T*)residual, w, w_f32, (T*)stream_out, (T*)out, hidden, eps);
 }
 
 TK_API int tk_rmsnorm(int dt, const void* x, const void* w, int w_f32, void* out, int rows,
@@ -66,12 +174,26 @@ TK_API int tk_rmsnorm(int dt, const void* x, const void* w, int w_f32, void* out
   TK_REQUIRE(rows >= 0 && hidden > 0, "rmsnorm: bad sizes %d %d", rows, hidden);
   if (rows == 0) return 0;
   if (dt == TK_F32)
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)x, w,
-                       w_f32, (float*)out, hidden, eps);
+    launch_rmsnorm<float, false>(x, nullptr, w, w_f32, nullptr, out, rows, hidden, eps, stream);
   else
-    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)x,
-                       w, w_f32, (bf16_t*)out, hidden, eps);
+    launch_rmsnorm<bf16_t, false>(x, nullptr, w, w_f32, nullptr, out, rows, hidden, eps, stream);
   TK_CHECK_LAUNCH("rmsnorm");
+  return 0;
+}
+
+// stream_out = x + residual (rounded); out = RMSNorm(stream_out) * w.  Four buffers, none shared.
+TK_API int tk_add_rmsnorm(int dt, const void* x, const void* residual, const void* w, int w_f32,
+                          void* stream_out, void* out, int rows, int hidden, float eps, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes %d %d", rows, hidden);
+  TK_REQUIRE(x && residual && stream_out && out && w, "add_rmsnorm: an operand is missing");
+  TK_REQUIRE(out != x && out != residual && out != stream_out && stream_out != x && stream_out != residual,
+             "add_rmsnorm: inputs and outputs must not share a buffer");
+  if (rows == 0) return 0;
+  if (dt == TK_F32)
+    launch_rmsnorm<float, true>(x, residual, w, w_f32, stream_out, out, rows, hidden, eps, stream);
+  else
+    launch_rmsnorm<bf16_t, true>(x, residual, w, w_f32, stream_out, out, rows, hidden, eps, stream);
+  TK_CHECK_LAUNCH("add_rmsnorm");
   return 0;
 }
 
@@ -81,26 +203,55 @@ TK_API int tk_rmsnorm(int dt, const void* x, const void* w, int w_f32, void* out
 // --------------------------------------------------------------------------
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
-  const T* g = gu + (size_t)blockIdx.x * 2 * inter;
+  const T* g = gu + (size_t)blockIdx.y * 2 * inter;
   const T* u = g + inter;
-  T* o = out + (size_t)blockIdx.x * inter;
-  for (int i = threadIdx.x; i < inter; i += blockDim.x) {
+  T* o = out + (size_t)blockIdx.y * inter;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < inter) {
     float gv = to_f32<T>(g[i]);
     float s = round_to<T>(gv / (1.0f + expf(-gv)));
     o[i] = from_f32<T>(s * to_f32<T>(u[i]));
   }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_packed_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+  constexpr int N = Pack<T>::N;
+  const int piece = blockIdx.x * blockDim.x + threadIdx.x;
+  if (piece >= inter / N) return;
+  const T* g = gu + (size_t)blockIdx.y * 2 * inter + (size_t)piece * N;
+  Pack<T> gv, uv, o;
+  gv.load(g);
+  uv.load(g + inter);
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float x = to_f32<T>(gv.v[j]);
+    const float s = round_to<T>(x / (1.0f + expf(-x)));
+    o.v[j] = from_f32<T>(s * to_f32<T>(uv.v[j]));
+  }
+  o.store(out + (size_t)blockIdx.y * inter + (size_t)piece * N);
+}
+
+template <typename T>
+static void launch_swiglu(const void* gate_up, void* out, int rows, int inter, hipStream_t stream) {
+  constexpr int N = Pack<T>::N;
+  if (inter % N == 0 && aligned16(gate_up) && aligned16(out))
+    hipLaunchKernelGGL(swiglu_packed_kernel<T>, dim3((inter / N + 255) / 256, rows), dim3(256), 0, stream,
+                       (const T*)gate_up, (T*)out, inter);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<T>, dim3((inter + 255) / 256, rows), dim3(256), 0, stream,
+                       (const T*)gate_up, (T*)out, inter);
+}
+
 TK_API int tk_swiglu(int dt, const void* gate_up, void* out, int rows, int inter,
                          hipStream_t stream) {
   TK_REQUIRE(rows >= 0 && inter > 0, "swiglu: bad sizes %d %d", rows, inter);
+  TK_REQUIRE(rows < 65536, "swiglu: %d rows are too many for one call", rows);
   if (rows == 0) return 0;
   if (dt == TK_F32)
-    hipLaunchKernelGGL(swiglu_kernel<float>, dim3(rows), dim3(256), 0, stream,
-                       (const float*)gate_up, (float*)out, inter);
+    launch_swiglu<float>(gate_up, out, rows, inter, stream);
   else
-    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream,
-                       (const bf16_t*)gate_up, (bf16_t*)out, inter);
+    launch_swiglu<bf16_t>(gate_up, out, rows, inter, stream);
   TK_CHECK_LAUNCH("swiglu");
   return 0;
 }

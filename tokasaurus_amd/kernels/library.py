@@ -24,6 +24,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
     "core": {
         "tk_embed_gather": [c_int, _P, _P, _P, _P, c_int, c_int, c_int, _P],
         "tk_rmsnorm": [c_int, _P, _P, c_int, _P, c_int, c_int, c_float, _P],
+        "tk_add_rmsnorm": [c_int, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_float, _P],
         "tk_swiglu": [c_int, _P, _P, c_int, c_int, _P],
         "tk_gather_rows": [c_int, _P, c_int, _P, _P, c_int, c_int, _P],
         "tk_rope_table": [_P, _P, _P, c_int, c_int, _P],

@@ -124,6 +124,21 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
+def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """(x + residual rounded to the storage type, its RMSNorm times ``weight``) in one pass."""
+    _gpu(x, residual, weight)
+    _need(x.dim() == 2 and x.is_contiguous() and residual.shape == x.shape and residual.is_contiguous()
+          and residual.dtype == x.dtype, "add_rmsnorm: x and residual must be contiguous [rows, H] of one type")
+    rows, hidden = x.shape
+    _need(weight.shape == (hidden,) and weight.is_contiguous() and weight.dtype in (x.dtype, torch.float32),
+          f"add_rmsnorm: the weight must be [H] of {x.dtype} or float32")
+    stream_out, out = torch.empty_like(x), torch.empty_like(x)
+    w_f32 = 1 if (weight.dtype == torch.float32 and x.dtype != torch.float32) else 0
+    call("tk_add_rmsnorm", dtype_code(x.dtype), x.data_ptr(), residual.data_ptr(), weight.data_ptr(), w_f32,
+         stream_out.data_ptr(), out.data_ptr(), rows, hidden, float(eps), _stream())
+    return stream_out, out
+
+
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """[rows, 2I] laid out [gate | up] -> silu(gate) * up, [rows, I]."""
     _gpu(gate_up)

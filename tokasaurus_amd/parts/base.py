@@ -115,12 +115,14 @@ class StepContext:
 
 @dataclass
 class Prepared:
-    """What the product in front of a norm has already done for it (the rows times the
-    norm's weight, and partial sums of their squares): ``data`` is the kernels' own
-    record (``kernels.ops.Prenorm``), ``norm`` the norm it was made for."""
+    """What the product in front of a norm has already done for it, and the norm it did it
+    for: either ``data``, the kernels' own record (``kernels.ops.Prenorm``: the rows times
+    the norm's weight and partial sums of their squares, which the next product folds in),
+    or ``normed``, the normed rows themselves (made in the pass that added the residual)."""
 
     data: Any
     norm: "Norm"
+    normed: torch.Tensor | None = None
 
 
 @dataclass
@@ -135,10 +137,15 @@ class Normed:
     prepared: Prepared | None = None
 
     def usable(self) -> Prepared | None:
+        """The record a product can fold in, if it was made for this very norm."""
         p = self.prepared
-        return p if p is not None and p.norm is self.norm and getattr(self.norm, "fusable_rms", False) else None
+        ok = p is not None and p.data is not None and p.norm is self.norm and getattr(self.norm, "fusable_rms", False)
+        return p if ok else None
 
     def materialize(self) -> torch.Tensor:
+        p = self.prepared
+        if p is not None and p.normed is not None and p.norm is self.norm:
+            return p.normed
         return self.norm.forward(self.x)
 
 

@@ -89,8 +89,8 @@ class PreNormBlock(Block):
             out = self.mixer.forward(Normed(x, self.mixer_norm, prepared), residual, ctx, cache, state, rows,
                                      emit_norm=self.ff_norm)
         else:
-            out = self.mixer.forward(self.mixer_norm.forward(x), residual, ctx, cache, state, rows)
+            out = self.mixer.forward(Normed(x, self.mixer_norm, prepared).materialize(), residual, ctx, cache, state, rows)
         x, prepared = stream_and_prepared(out)
         if self.feed_forward.fuses_norm:
             return self.feed_forward.forward(Normed(x, self.ff_norm, prepared), x, emit_norm=next_norm)
-        return self.feed_forward.forward(self.ff_norm.forward(x), x)
+        return self.feed_forward.forward(Normed(x, self.ff_norm, prepared).materialize(), x)

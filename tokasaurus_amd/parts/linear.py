@@ -116,6 +116,10 @@ class Linear:
         if emit_norm is not None and getattr(emit_norm, "fusable_rms", False) and self._fast(x.shape[0]):
             out, data = ops.gemm_skinny_bf16(x, self.weight, residual=residual, emit_weight=emit_norm.weight)
             return out, Prepared(data, emit_norm)
+        if emit_norm is not None and getattr(emit_norm, "fusable_rms", False) and x.shape[0] > 0:
+            # one pass adds the residual and norms the sum
+            out, normed = ops.add_rmsnorm(self(x), residual.contiguous(), emit_norm.weight, emit_norm.eps)
+            return out, Prepared(None, emit_norm, normed)
         return self(x, residual=residual), None
 
     def rope_append(self, x: torch.Tensor | Normed, rope: "ops.RopeAppend") -> torch.Tensor | None:
