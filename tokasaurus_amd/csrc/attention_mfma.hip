@@ -389,41 +389,57 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
 // Adds the partial results of split tiles, always in split order.  One wavefront
 // per (tile, kv head, row): lane i takes the statistics of split i (of splits i, i + 64, ..),
 // then every lane sums one (or more) of the row's d outputs over the splits, with the
-// weights handed from lane to lane.
+// weights handed from lane to lane.  Where the partial results lie depends on the launch
+// alone, so the first MG_AHEAD splits are loaded before the tile's range (which says how
+// many of them count) has arrived: the kernel is little more than one trip to memory.
+#define MG_AHEAD 16
 __global__ __launch_bounds__(256) void attention_merge_kernel(AttnArgs a, int D, int row_tiles) {
   const int tile = blockIdx.x, kvh = blockIdx.y;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.z * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int rows_per_tile = 16 * row_tiles;
+  const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
+  const float* ml = a.part_ml + (item0 * rows_per_tile + row) * 2;  // split sp is sp * rows_per_tile * 2 further
+  const size_t ml_step = (size_t)rows_per_tile * 2;
+  const float* po = a.part_o + (item0 * rows_per_tile + row) * D;
+  const size_t po_step = (size_t)rows_per_tile * D;
+  // ahead of everything: what may be stale or never written is not used below
+  float ahead[MG_AHEAD];
+  const int d_first = min(lane, D - 1);
+#pragma unroll
+  for (int sp = 0; sp < MG_AHEAD; ++sp) ahead[sp] = sp < a.max_splits ? po[sp * po_step + d_first] : 0.f;
+  float ms_own = -INFINITY, ls_own = 0.f;
+  if (lane < a.max_splits) {
+    ms_own = ml[lane * ml_step];
+    ls_own = ml[lane * ml_step + 1];
+  }
+
   const TileRange t = tile_range(a, tile, row_tiles);
   const int nsp = t.s_last - t.s_first + 1;
   if (nsp == 1) return;
   const int base = row < 16 ? t.row0[0] : t.row0[1];
   const int flat = base + (row & 15);
   if (base < 0 || flat >= t.n_rows) return;
-  const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
-  const float* ml = a.part_ml + (item0 * rows_per_tile + row) * 2;  // split sp is sp * rows_per_tile * 2 further
-  const size_t ml_step = (size_t)rows_per_tile * 2;
-  const float* po = a.part_o + (item0 * rows_per_tile + row) * D;
-  const size_t po_step = (size_t)rows_per_tile * D;
   const int tok = flat / a.group, g = flat - tok * a.group;
   bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
-  float m = -INFINITY;
-  for (int sp = lane; sp < nsp; sp += 64) m = fmaxf(m, ml[sp * ml_step]);
+  if (lane >= nsp) ms_own = -INFINITY;
+  float m = ms_own;
+  for (int sp = lane + 64; sp < nsp; sp += 64) m = fmaxf(m, ml[sp * ml_step]);
   m = wave_max(m);
   if (nsp <= 64) {
-    float w = 0.f, l = 0.f;
-    if (lane < nsp) {
-      const float ms = ml[lane * ml_step];
-      w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - m);
-      l = w * ml[lane * ml_step + 1];
-    }
-    const float inv = 1.0f / wave_sum(l);
+    const float w = ms_own == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms_own - m);
+    const float inv = 1.0f / wave_sum(lane < nsp ? w * ls_own : 0.f);
     for (int d0 = 0; d0 < D; d0 += 64) {  // every lane stays in the loop: the weights come from all of them
       const int d = min(d0 + lane, D - 1);
       float o = 0.f;
+#pragma unroll
+      for (int sp = 0; sp < MG_AHEAD; ++sp) {
+        const float ws = __shfl(w, sp, 64);
+        const float v = d0 == 0 ? ahead[sp] : (sp < nsp ? po[sp * po_step + d] : 0.f);
+        if (sp < nsp) o += ws * v;
+      }
 #pragma unroll 8
-      for (int sp = 0; sp < nsp; ++sp) o += __shfl(w, sp, 64) * po[sp * po_step + d];
+      for (int sp = MG_AHEAD; sp < nsp; ++sp) o += __shfl(w, sp, 64) * po[sp * po_step + d];
       if (d0 + lane < D) op[d] = __float2bfloat16(o * inv);
     }
     return;
