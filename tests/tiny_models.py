@@ -85,14 +85,14 @@ CONFIG_C = {
 }
 PAGE_C = 16
 
-# awkward sizes: no grouping (as many kv heads as heads), an intermediate size that is no
+# awkward sizes: a head size of 48, no grouping (as many kv heads as heads), an intermediate size that is no
 # multiple of 8 (the bfloat16 matrix-core products cannot take it: the plain kernel does),
 # an odd vocabulary, one layer, a large eps, pages of 32
 CONFIG_D = {
     "architectures": ["LlamaForCausalLM"],
     "model_type": "llama",
     "num_hidden_layers": 1,
-    "hidden_size": 80,
+    "hidden_size": 240,
     "num_attention_heads": 5,
     "num_key_value_heads": 5,
     "intermediate_size": 172,
