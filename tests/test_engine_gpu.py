@@ -128,6 +128,17 @@ def test_finishing_on_an_end_token_and_on_length(folders, tmp_path):
     assert ignore.tokens == free_run and ignore.finish_reason == "length"
     one = engine.generate([prompt], SamplingParams(max_tokens=1, ignore_eos=True))[0]  # ends in its prefill step
     assert one.tokens == free_run[:1] and engine.runner.manager.requests == {}
+    # a loop that waits for every step's tokens and one that launches the next step first
+    # (it finds the end token a step late) give the same completions
+    prompts = [random_tokens(n, cfg["vocab_size"], 70 + n) for n in (9, 5, 12, 7, 3, 10)]
+    params = [SamplingParams(temperature=0.9, max_tokens=24, seed=i) for i in range(len(prompts))]
+    runs = []
+    for ahead in (0, 8):
+        engine = Engine(EngineConfig(model=str(folder), dtype="float32", page_size=PAGE_A, kv_cache_num_tokens=512,
+                                     max_seqs_per_forward=3, scheduling_steps_ahead=ahead))
+        runs.append([(c.tokens, c.finish_reason) for c in engine.generate(prompts, params)])
+        assert engine.runner.manager.requests == {} and not engine.has_work()
+    assert runs[0] == runs[1]
 
 
 def test_pages_run_out_and_the_newest_request_starts_again(folders):

@@ -202,3 +202,74 @@ def test_random_workloads_finish_with_every_page_back(seed, optimistic):
         assert s.num_bumps == 0
     assert cache.num_free_pages() == [total] and cache.slots.num_free == cache.slots.num_slots
     cache.check()
+
+
+def drive(s, token_of, ahead):
+    """The engine's loop with a fake model: with ``ahead`` the next step is scheduled and
+    advanced before the tokens of the step before are resolved."""
+    finished, inflight, steps = {}, None, 0
+    while s.has_work() or inflight is not None:
+        d = s.schedule()
+        launched = None
+        if not d.empty():
+            toks = [token_of(r, r.sampled) for r in d.requests_with_output()]
+            s.advance(d)
+            launched = (d, toks)
+        if inflight is not None:
+            for r in s.resolve(inflight[0], inflight[1], [0.0] * len(inflight[1])):
+                finished[r.id] = (list(r.completion), r.finish_reason)
+            inflight = None
+        if launched is not None:
+            if ahead:
+                inflight = launched
+            else:
+                for r in s.resolve(launched[0], launched[1], [0.0] * len(launched[1])):
+                    finished[r.id] = (list(r.completion), r.finish_reason)
+        steps += 1
+        assert steps < 4000
+    return finished
+
+
+@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("optimistic", [False, True])
+def test_a_step_ahead_gives_the_completions_of_the_waiting_loop(seed, optimistic):
+    """Tokens are a function of (request, index) as with a real model: scheduling the
+    next step before the last one's tokens are back (end tokens are then found a step
+    late, a request may start again meanwhile) changes no completion, and every page
+    and slot comes back."""
+    def workload():
+        rng = random.Random(seed)
+        P = rng.choice([2, 4, 16])
+        s, cache = make(num_pages=rng.choice([24, 40]), page_size=P, max_tokens_per_forward=rng.choice([8, 24]),
+                        max_seqs=rng.choice([2, 4, 8]), optimistic=optimistic, eos=(3,))
+        total = cache.num_free_pages()[0]
+        for i in range(14):
+            plen, mt = rng.randint(1, 20), rng.randint(1, 12)
+            if math.ceil((plen + mt - 1) / P) <= total:
+                s.submit(req(f"r{i}", plen, mt, ignore_eos=(i % 5 == 0)))
+        return s, cache
+
+    def token_of(r, index):
+        return random.Random(f"{seed}/{r.id}/{index}").choice([3, 5, 6, 7, 8, 9])
+
+    results = []
+    for ahead in (False, True):
+        s, cache = workload()
+        total = cache.num_free_pages()
+        results.append(drive(s, token_of, ahead))
+        assert cache.num_free_pages() == total and cache.slots.num_free == cache.slots.num_slots
+        cache.check()
+    assert results[0] == results[1] and len(results[0]) > 0
+    assert any(reason == "stop" for _, reason in results[0].values())
+
+
+def test_an_end_token_found_a_step_late_costs_one_token_and_no_more():
+    s, cache = make(eos=(3,))
+    s.submit(req("a", 4, 10))
+    d0 = s.schedule(); s.advance(d0)                 # the prompt; its token is not back yet
+    d1 = s.schedule(); s.advance(d1)                 # scheduled ahead: a decodes once more
+    assert [r.id for r in d1.decode] == ["a"]
+    done = s.resolve(d0, [3], [0.0])                 # the first token was the end token
+    assert [r.id for r in done] == ["a"] and done[0].completion == [3] and done[0].finish_reason == "stop"
+    assert cache.num_free_pages() == [64] and not s.has_work()
+    assert s.resolve(d1, [7], [0.0]) == [] and done[0].completion == [3]  # dropped

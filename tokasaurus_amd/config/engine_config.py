@@ -47,6 +47,11 @@ class EngineConfig:
     hipgraph_max_size: int = 128
     hipgraph_step: int = 16
 
+    # --- steps launched before their tokens are back (tokasaurus/common_types.py:89; the
+    # reference queues up to 8 between two processes, this loop keeps at most one ahead:
+    # 0 waits for every step's tokens, anything above launches the next step first)
+    scheduling_steps_ahead: int = 8
+
     # --- debugging (tokasaurus/common_types.py:124-125)
     allocator_sanity_checks: bool = False
     bump_city_population_me: bool = False
@@ -75,6 +80,8 @@ class EngineConfig:
         for name in ("page_size", "kv_cache_num_tokens", "max_tokens_per_forward", "max_seqs_per_forward"):
             if getattr(self, name) <= 0:
                 raise OptionError(f"{name} must be positive")
+        if self.scheduling_steps_ahead < 0:
+            raise OptionError("scheduling_steps_ahead must not be negative")
         self.kv_cache_num_blocks()
         if self.max_num_tokens_per_request is None and max_position_embeddings is not None:
             self.max_num_tokens_per_request = min(max_position_embeddings, self.kv_cache_num_tokens)

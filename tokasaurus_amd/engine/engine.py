@@ -20,7 +20,7 @@ import torch
 
 from tokasaurus_amd.config.engine_config import EngineConfig
 from tokasaurus_amd.engine.batch import StepEntry
-from tokasaurus_amd.engine.runner import ModelRunner, Sampling
+from tokasaurus_amd.engine.runner import ModelRunner, Sampling, StepOutput
 from tokasaurus_amd.engine.scheduler import Decision, Request, Scheduler
 from tokasaurus_amd.sampling import SamplingParams, uniform_for
 
@@ -102,6 +102,7 @@ class Engine:
         self.stats = Stats()
         self._next_id = 0
         self._request_seed: dict[str, int] = {}
+        self._inflight: tuple[Decision, StepOutput] | None = None  # launched, its tokens not read yet
 
     # ---- requests
     def submit(self, prompt: list[int], params: SamplingParams | None = None, request_id: str | None = None) -> str:
@@ -122,7 +123,7 @@ class Engine:
         return self.scheduler.abort(request_id) is not None
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._inflight is not None
 
     # ---- one step of the loop
     def _entries(self, decision: Decision) -> list[StepEntry]:
@@ -134,38 +135,60 @@ class Engine:
             entries.append(StepEntry(req.id, None, [0]))  # the token comes from the request's slot
         return entries
 
-    def step(self) -> list[Completion]:
-        """Schedule, run and sample one batch; returns the requests that finished."""
-        t0 = time.perf_counter()
+    def _launch(self) -> "tuple[Decision, StepOutput] | None":
+        """Schedule a batch, start it on the device and make the changes that do not
+        depend on its tokens; None when there is nothing to run."""
         decision = self.scheduler.schedule()
         self.stats.bumps = self.scheduler.num_bumps
         if decision.empty():
-            if self.scheduler.queued:
-                raise RuntimeError("requests are queued but none can be admitted: the cache is too small for them")
-            return []
+            return None
         out_reqs = decision.requests_with_output()
         # the rows of the step's output follow the entries: prompts that end, then decodes
         temps = [r.params.temperature for r in out_reqs]
         us = [
-            uniform_for(self.config.seed, self._request_seed[r.id], len(r.completion)) if r.params.temperature > 0 else 0.0
+            uniform_for(self.config.seed, self._request_seed[r.id], r.sampled) if r.params.temperature > 0 else 0.0
             for r in out_reqs
         ]
         out = self.runner.run(self._entries(decision), Sampling(temps, us))
-        tokens: list[int] = []
-        logprobs: list[float] | None = None
-        if out_reqs:
-            tokens = out.ids.tolist()  # the step's one device-to-host synchronisation
-            if self.config.enable_chosen_logprobs and out.logprobs is not None:
-                logprobs = out.logprobs.tolist()
-        finished = self.scheduler.apply(decision, tokens, logprobs)
+        self.scheduler.advance(decision)
         self.stats.steps += 1
         self.stats.prefill_tokens += sum(n for _, n in decision.prefill)
         self.stats.decode_tokens += len(decision.decode)
-        self.stats.seconds += time.perf_counter() - t0
+        return decision, out
+
+    def _collect(self, launched: "tuple[Decision, StepOutput]") -> list[Completion]:
+        """Wait for a launched step's tokens (the loop's one wait for the device) and
+        hand them to the scheduler; the requests that are finished with it."""
+        decision, out = launched
+        tokens, logprobs = out.sampled()
+        keep_logprobs = self.config.enable_chosen_logprobs and out.logprobs is not None
+        finished = self.scheduler.resolve(decision, tokens, logprobs if keep_logprobs else None)
         done = []
         for r in finished:
             self._request_seed.pop(r.id, None)
             done.append(Completion(r.id, r.prompt, list(r.completion), list(r.logprobs), r.finish_reason or "", r.times_bumped))
+        return done
+
+    def step(self) -> list[Completion]:
+        """Launch one batch and return the requests that finished.  With
+        ``scheduling_steps_ahead`` above 0 the batch is launched before the tokens of the
+        one before are read, so the device does not wait while the host schedules: the
+        completions returned are those of the batch before.  A request that stops at an end
+        token is found out one step late and has one token computed for nothing."""
+        t0 = time.perf_counter()
+        done: list[Completion] = []
+        launched = self._launch()
+        if self._inflight is not None:
+            done = self._collect(self._inflight)
+            self._inflight = None
+        if launched is None:
+            if not done and self.scheduler.queued and not self.scheduler.running():
+                raise RuntimeError("requests are queued but none can be admitted: the cache is too small for them")
+        elif self.config.scheduling_steps_ahead > 0:
+            self._inflight = launched
+        else:
+            done += self._collect(launched)
+        self.stats.seconds += time.perf_counter() - t0
         return done
 
     def run_until_done(self) -> list[Completion]:

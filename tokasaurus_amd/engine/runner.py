@@ -48,6 +48,20 @@ class StepOutput:
     logits: torch.Tensor  # [wanted, vocab] float32
     ids: torch.Tensor | None = None  # [wanted] int32, when the step sampled
     logprobs: torch.Tensor | None = None
+    # a sampled step also copies ids and log-probabilities to pinned host memory, in stream
+    # order right behind the step: they can be read while later steps already run
+    host: torch.Tensor | None = None  # [2, >= wanted] int32 (row 1 holds the bits of float32)
+    ready: torch.cuda.Event | None = None
+
+    def sampled(self) -> tuple[list[int], list[float]]:
+        """Token ids and their log-probabilities on the host; waits for this step only."""
+        if self.ids is None:
+            return [], []
+        n = self.ids.shape[0]
+        if self.host is None:
+            return self.ids.tolist(), (self.logprobs.tolist() if self.logprobs is not None else [])
+        self.ready.synchronize()
+        return self.host[0, :n].tolist(), self.host[1, :n].view(torch.float32).tolist()
 
 
 def graph_buckets(max_size: int, step: int) -> list[int]:
@@ -232,6 +246,8 @@ class ModelRunner:
             self.graph_sizes.sort()
         self.recorded: dict[tuple[int, int], RecordedDecodeStep] = {}  # by (rows, context bound)
         self.graph_pool = torch.cuda.graph_pool_handle() if use_graphs else None
+        self._host_ring: list[tuple[torch.Tensor, torch.cuda.Event]] = []  # pinned buffers for sampled ids
+        self._host_at = 0
         self.storage = CacheStorage(
             self.groups,
             [num_pages] * len(self.groups),
@@ -358,9 +374,26 @@ class ModelRunner:
                 out.ids, out.logprobs = ops.sample(
                     logits, params[0], params[1], slot_t, self.storage.last_token if write_slots else None
                 )
+        if out.ids is not None and out.ids.shape[0] > 0:
+            self._copy_to_host(out)
         for e in planned:
             self.manager.advance(e.request_id, e.start + e.q_len)
         return out
+
+    def _copy_to_host(self, out: StepOutput) -> None:
+        n = out.ids.shape[0]
+        if not self._host_ring or self._host_ring[0][0].shape[1] < n:
+            width = max(n, self.manager.slots.num_slots)
+            self._host_ring = [(torch.zeros((2, width), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                               for _ in range(4)]
+        buf, event = self._host_ring[self._host_at % len(self._host_ring)]
+        self._host_at += 1
+        event.synchronize()  # whoever used this buffer four steps ago has long read it
+        buf[0, :n].copy_(out.ids, non_blocking=True)
+        if out.logprobs is not None:
+            buf[1, :n].view(torch.float32).copy_(out.logprobs, non_blocking=True)
+        event.record()
+        out.host, out.ready = buf, event
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         """Run one batch and return its logits only (nothing is sampled or written to slots)."""

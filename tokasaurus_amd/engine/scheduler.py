@@ -45,13 +45,15 @@ class Request:
     logprobs: list[float] = field(default_factory=list)
     finish_reason: str | None = None
     times_bumped: int = 0
+    sampled: int = 0  # completion tokens sampled so far, those whose ids have not come back included
+    epoch: int = 0  # grows when the request starts again: results of steps from before are dropped
 
     def max_cache_tokens(self) -> int:
         return len(self.prompt) + self.params.max_tokens - 1
 
     def cache_tokens(self) -> int:
         """Tokens in the cache: the prompt part done plus every completion token fed back."""
-        return self.prompt_done + max(0, len(self.completion) - 1) if self.state == DECODING else self.prompt_done
+        return self.prompt_done + max(0, self.sampled - 1) if self.state == DECODING else self.prompt_done
 
 
 @dataclass
@@ -60,6 +62,7 @@ class Decision:
 
     prefill: list[tuple[Request, int]]
     decode: list[Request]
+    outputs: list[tuple[Request, int]] = field(default_factory=list)  # set by advance: (request, its epoch then)
 
     def num_tokens(self) -> int:
         return sum(n for _, n in self.prefill) + len(self.decode)
@@ -186,6 +189,8 @@ class Scheduler:
         req.state, req.prompt_done = QUEUED, 0
         req.completion.clear()
         req.logprobs.clear()
+        req.sampled = 0
+        req.epoch += 1
         req.times_bumped += 1
         self.num_bumps += 1
         self.queued[req.id] = req
@@ -212,13 +217,15 @@ class Scheduler:
             req.state = PREFILLING
             self.prefilling[req.id] = req
 
-    # ---- after the step ran
-    def apply(self, decision: Decision, tokens: list[int], logprobs: list[float] | None = None) -> list[Request]:
-        """Advance every request of the decision; ``tokens`` are the sampled
-        tokens in the order of ``decision.requests_with_output()``.  Returns the
-        requests that finished; their pages and slots are free on return."""
+    # ---- after the step was launched, and after its tokens came back
+    def advance(self, decision: Decision) -> None:
+        """What a step changes whatever its tokens turn out to be: prompt progress, a
+        prompt's end, one more sampled token for every request with output, and the end of
+        a request by length (its pages and slot are free on return: a later step runs
+        after this one on the device, so it may have them).  With this done the next step
+        can be scheduled and launched before this step's tokens have come back
+        (the reference schedules ahead likewise, tokasaurus/manager/manager.py:999-1008)."""
         out_reqs = decision.requests_with_output()
-        assert len(tokens) == len(out_reqs), (len(tokens), len(out_reqs))
         for req, n in decision.prefill:
             req.prompt_done += n
             self.cache.advance(req.id, req.prompt_done)
@@ -228,22 +235,44 @@ class Scheduler:
                 self.decoding[req.id] = req
         for req in decision.decode:
             # the token fed in this step (the one sampled before) is now in the cache
-            self.cache.advance(req.id, req.prompt_done + len(req.completion))
+            self.cache.advance(req.id, req.prompt_done + req.sampled)
+        decision.outputs = [(req, req.epoch) for req in out_reqs]
+        for req in out_reqs:
+            req.sampled += 1
+            if req.sampled >= req.params.max_tokens:  # manager.py:201-204
+                self.decoding.pop(req.id)
+                self.cache.release(req.id)
+                req.state, req.finish_reason = FINISHED, "length"
+        if self.sanity_checks:
+            self.cache.check()
+
+    def resolve(self, decision: Decision, tokens: list[int], logprobs: list[float] | None = None) -> list[Request]:
+        """Take the sampled tokens of an advanced step, in the order of its requests with
+        output.  A token for a request that has meanwhile started again, was aborted or
+        stopped at an end token is dropped (it was computed for nothing).  Returns the
+        requests that are finished and have all their tokens."""
+        assert len(tokens) == len(decision.outputs), (len(tokens), len(decision.outputs))
         finished = []
-        for i, req in enumerate(out_reqs):
+        for i, (req, epoch) in enumerate(decision.outputs):
+            if req.epoch != epoch or req.finish_reason in ("abort", "stop"):
+                continue
             req.completion.append(int(tokens[i]))
             if logprobs is not None:
                 req.logprobs.append(float(logprobs[i]))
-            reason = None
-            if len(req.completion) >= req.params.max_tokens:
-                reason = "length"  # manager.py:201-204
-            if not req.params.ignore_eos and int(tokens[i]) in self.eos_token_ids:
-                reason = "stop"  # manager.py:205-206
-            if reason is not None:
-                self.decoding.pop(req.id)
-                self.cache.release(req.id)
-                req.state, req.finish_reason = FINISHED, reason
+            if not req.params.ignore_eos and int(tokens[i]) in self.eos_token_ids:  # manager.py:205-206
+                if req.state != FINISHED:
+                    self.decoding.pop(req.id)
+                    self.cache.release(req.id)
+                req.state, req.finish_reason = FINISHED, "stop"
+                req.sampled = len(req.completion)
+                finished.append(req)
+            elif req.state == FINISHED and len(req.completion) == req.sampled:
                 finished.append(req)
         if self.sanity_checks:
             self.cache.check()
         return finished
+
+    def apply(self, decision: Decision, tokens: list[int], logprobs: list[float] | None = None) -> list[Request]:
+        """advance and resolve in one: for a loop that waits for every step's tokens."""
+        self.advance(decision)
+        return self.resolve(decision, tokens, logprobs)
