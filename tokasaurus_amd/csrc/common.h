@@ -49,6 +49,13 @@ __host__ __device__ __forceinline__ size_t value_offset(int d, int in_page, int 
   return ((size_t)(in_page / TK_VALUE_QUAD) * d + e) * TK_VALUE_QUAD + (in_page % TK_VALUE_QUAD);
 }
 
+// One rotation of a pair by (cos, sin) in 32-bit, written out in fused multiply-adds so that
+// every kernel that rotates gets the same bits whatever the compiler would contract.
+__device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s, float& o1, float& o2) {
+  o1 = __fmaf_rn(x1, c, -__fmul_rn(x2, s));
+  o2 = __fmaf_rn(x2, c, __fmul_rn(x1, s));
+}
+
 template <typename T>
 __device__ __forceinline__ float to_f32(T v);
 template <>

@@ -335,8 +335,10 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
     T* x = row + h * d;
     const float x1 = to_f32<T>(x[j]), x2 = to_f32<T>(x[j + half]);
     const float cj = c ? c[j] : 1.f, sj = s ? s[j] : 0.f;
-    x[j] = from_f32<T>(x1 * cj - x2 * sj);
-    x[j + half] = from_f32<T>(x2 * cj + x1 * sj);
+    float o1, o2;
+    rotate_pair(x1, x2, cj, sj, o1, o2);
+    x[j] = from_f32<T>(o1);
+    x[j + half] = from_f32<T>(o2);
   }
   if (!write_cache) return;
 
@@ -349,8 +351,10 @@ __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
     const float x1 = to_f32<T>(krow[h * d + j]), x2 = to_f32<T>(krow[h * d + j + half]);
     const float cj = c ? c[j] : 1.f, sj = s ? s[j] : 0.f;
     T* dst = kcache + ((size_t)page * nkv + h) * P * d;
-    dst[key_offset(P, p, j)] = from_f32<T>(x1 * cj - x2 * sj);
-    dst[key_offset(P, p, j + half)] = from_f32<T>(x2 * cj + x1 * sj);
+    float o1, o2;
+    rotate_pair(x1, x2, cj, sj, o1, o2);
+    dst[key_offset(P, p, j)] = from_f32<T>(o1);
+    dst[key_offset(P, p, j + half)] = from_f32<T>(o2);
   }
   for (int i = threadIdx.x; i < nkv * d; i += blockDim.x) {
     const int h = i / d, e = i % d;

@@ -171,19 +171,41 @@ __device__ __forceinline__ void emit_for_norm(const GemmArgs& a, const float (&x
 
 // Rotation with append for 4 columns c .. c+3 of head h (and their partners c + d/2): x1, x2
 // are the products rounded to bfloat16 as a plain store would leave them.
-__device__ __forceinline__ void rope_store(const GemmArgs& a, f32x4_t s0, f32x4_t s1, int token, int h, int c) {
+// What the rotation of one unit (token, head h, columns c .. c+3) reads besides the products;
+// asked for before the main loop so that the epilogue does not wait for it.
+struct RopeOperands {
+  int pos, page;
+  float cs[4], sn[4];
+};
+
+__device__ __forceinline__ RopeOperands rope_operands(const GemmArgs& a, int token, int h, int c) {
+  RopeOperands r;
+  const int half = a.d >> 1;
+  const int t = min(token, a.M - 1);
+  r.pos = a.positions[t];
+  r.page = h >= a.nq ? a.block_table[(size_t)a.token_req[t] * a.table_stride + r.pos / a.P] : 0;
+  const bool rotate = h < a.nq + a.nkv && a.cos_t != nullptr;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const bool on = rotate && c + j < half;
+    r.cs[j] = on ? a.cos_t[(size_t)r.pos * half + c + j] : 1.f;
+    r.sn[j] = on ? a.sin_t[(size_t)r.pos * half + c + j] : 0.f;
+  }
+  return r;
+}
+
+__device__ __forceinline__ void rope_store(const GemmArgs& a, f32x4_t s0, f32x4_t s1, int token, int h, int c,
+                                           const RopeOperands& r) {
   if (token >= a.M) return;
   const int half = a.d >> 1;
-  const int pos = a.positions[token];
+  const int pos = r.pos;
   float o1[4], o2[4];
   const bool rotate = h < a.nq + a.nkv && a.cos_t != nullptr;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const float x1 = round_to<bf16_t>(s0[j]), x2 = round_to<bf16_t>(s1[j]);
     if (rotate && c + j < half) {
-      const float cj = a.cos_t[(size_t)pos * half + c + j], sj = a.sin_t[(size_t)pos * half + c + j];
-      o1[j] = x1 * cj - x2 * sj;
-      o2[j] = x2 * cj + x1 * sj;
+      rotate_pair(x1, x2, r.cs[j], r.sn[j], o1[j], o2[j]);
     } else {
       o1[j] = x1;
       o2[j] = x2;
@@ -199,7 +221,7 @@ __device__ __forceinline__ void rope_store(const GemmArgs& a, f32x4_t s0, f32x4_
       }
     return;
   }
-  const int page = a.block_table[(size_t)a.token_req[token] * a.table_stride + pos / a.P];
+  const int page = r.page;
   const int off = pos % a.P;
   if (h < a.nq + a.nkv) {
     bf16_t* dst = a.kcache + ((size_t)page * a.nkv + (h - a.nq)) * a.P * a.d;
@@ -264,6 +286,15 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) ap[mb] = a.A + (size_t)min(mb * 16 + r, a.M - 1) * a.lda + q * 8;
 
+  // what the rotation of this thread's first unit reads besides the sums (position, page,
+  // cos and sin) is asked for now, so that it has arrived when the main loop is through
+  constexpr int UNITS = (PAIRED ? 1 : NT) * MB * 64;
+  RopeOperands rope_pre = {};
+  if (EPI == EPI_ROPE && tid < UNITS) {
+    const int l0 = tid & 63, mb0 = (tid >> 6) % MB;
+    rope_pre = rope_operands(a, mb0 * 16 + (l0 & 15), rope_head, rope_col + (l0 >> 4) * 4);
+  }
+
   f32x4_t acc[NT][MB];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -323,7 +354,6 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
       for (int mb = 0; mb < MB; ++mb) red[(wave * NT * MB + t * MB + mb) * 64 + lane] = acc[t][mb];
   }
   if (WK > 1 || NORM) __syncthreads();
-  constexpr int UNITS = (PAIRED ? 1 : NT) * MB * 64;
   for (int u = tid; u < UNITS; u += blockDim.x) {
     const int l = u & 63, mb = (u >> 6) % MB, t = (u >> 6) / MB;
     const int token = mb * 16 + (l & 15), qq = l >> 4;
@@ -346,7 +376,9 @@ __global__ __launch_bounds__(SK_MAX_WAVES * 64) void gemm_skinny_kernel(GemmArgs
     const float scale = NORM ? scales[token] : 1.0f;
     const bool live = qq * 4 < TH && token < a.M;
     if (EPI == EPI_ROPE) {
-      if (live) rope_store(a, s0 * scale, s1 * scale, token, rope_head, rope_col + qq * 4);
+      if (live)
+        rope_store(a, s0 * scale, s1 * scale, token, rope_head, rope_col + qq * 4,
+                   u == tid ? rope_pre : rope_operands(a, token, rope_head, rope_col + qq * 4));
     } else {
       const int tile = PAIRED ? g : g * NT + t;
       const int n = tile * TH + qq * 4;
