@@ -101,6 +101,16 @@ __device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int
   return t;
 }
 
+// first <= x <= last as one unsigned comparison (an empty range, last < first, holds nothing)
+struct Range {
+  int first;
+  unsigned span;
+  __device__ __forceinline__ bool holds(int x) const { return (unsigned)(x - first) <= span; }
+};
+__device__ __forceinline__ Range range_of(int first, int last) {
+  return last >= first ? Range{first, (unsigned)(last - first)} : Range{0x7fffffff, 0u};
+}
+
 // The maximum over the four lanes (r, 0..3) that share a row: lanes 16 and 32 apart,
 // with the gfx950 swaps of 16-lane rows and of wavefront halves.
 __device__ __forceinline__ float max_over_quarters(float x) {
@@ -125,24 +135,40 @@ struct StepRegs {
 
 // BIG: pages of 16 keys or more, so the 16 keys of a block lie in one page, which a
 // scalar load looks up; the lane's part of the address is the same in every step.
+// The pages of the two 16-key blocks of the step at `kb` (BIG only): looked up a step before
+// the loads that need them are issued, so that no load waits for a table entry.
+struct StepPages {
+  int page[2];
+};
+
+__device__ __forceinline__ StepPages step_pages(const AttnArgs& a, const int* table, int kb, int lo, int hi) {
+  const int sh = a.p_shift;
+  StepPages p;
+  p.page[0] = table[min(max(kb >> sh, lo >> sh), hi >> sh)];
+  p.page[1] = table[min(max((kb + 16) >> sh, lo >> sh), hi >> sh)];
+  return p;
+}
+
 template <int DT, bool BIG>
-__device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, const int* table,
+__device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, const int* table, const StepPages& pages,
                                           int kvh, int kb, int lo, int hi, int r, int q) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
   const int P = a.P, sh = a.p_shift;
+  // the lane's own part of a key and of a value address inside any page of this kv head
+  const unsigned lane_k = (unsigned)(kvh * P * D + r * 8);
+  const unsigned lane_v = (unsigned)(kvh * P * D + (q * D + r) * 4);
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
     const bf16_t* kp;
     const bf16_t* vp;
     if constexpr (BIG) {
       const int key0 = kb + blk * 16;
-      const int pidx = min(max(key0 >> sh, lo >> sh), hi >> sh);
-      const int page = table[pidx];
-      const size_t base = ((size_t)page * a.nkv + kvh) * ((size_t)P * D);
+      // one 32 x 32 -> 64-bit product a page: the kv head's offset is in the lane's part already
+      const size_t base = (size_t)(unsigned)pages.page[blk] * (unsigned)(a.nkv * P * D);
       const int in_page = key0 & (P - 1);
-      kp = a.kcache + base + (size_t)(in_page + r) * 8;
-      vp = a.vcache + base + (size_t)(in_page >> 2) * (D * 4) + (size_t)(q * D + r) * 4;
+      kp = a.kcache + base + (unsigned)(in_page * 8) + lane_k;
+      vp = a.vcache + base + (unsigned)((in_page >> 2) * (D * 4)) + lane_v;
     } else {
       const int kk = min(max(kb + blk * 16 + r, lo), hi);
       const int page = table[kk >> sh];
@@ -193,6 +219,16 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
   const int k_end = min(t.hi + 1, s * a.split + (wave + 1) * sub);
   const int* table = a.block_table + (size_t)t.req * a.table_stride;
 
+  // the steps (by their first key) in which a row tile has a row that sees a key, in which all
+  // of its rows see all 32 keys, and in which all 32 keys lie in the tile's range
+  Range active[RT], unmasked[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    active[rt] = range_of(t.rt_lo[rt] - 31, t.rt_hi[rt]);
+    unmasked[rt] = range_of(t.full_lo[rt], t.full_hi[rt] - 31);
+  }
+  const Range inside = range_of(t.lo, t.hi - 31);
+
   // this lane's row in each of the RT tiles
   int pos_r[RT], lo_r[RT], flat_r[RT];
   bf16x8_t qv[RT][KS];
@@ -230,7 +266,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
   }
 
   auto compute_step = [&](StepRegs<DT>& cur, const int kb) {
-    if (kb < t.lo || kb + 31 > t.hi) {
+    if (!inside.holds(kb)) {
       // values of keys outside the tile's range may be anything (a freed page): make them
       // zero by masking their 16 bits
       uint32_t keep[4];
@@ -250,7 +286,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      if (kb > t.rt_hi[rt] || kb + 31 < t.rt_lo[rt]) continue;  // none of the tile's rows sees these keys
+      if (!active[rt].holds(kb)) continue;  // none of the tile's rows sees these keys
       f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -262,7 +298,7 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
       float sc[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) sc[e] = st[e >> 2][e & 3];
-      if (kb < t.full_lo[rt] || kb + 31 > t.full_hi[rt]) {
+      if (!unmasked[rt].holds(kb)) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int key = kb + (e >> 2) * 16 + q * 4 + (e & 3);
@@ -298,16 +334,26 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
   };
 
   StepRegs<DT> ring[PF];
+  // With two row tiles (prompts: many steps a wavefront) the pages of a step are looked up when
+  // the loads of the step before are issued; with one (decode: few steps) right before its own.
+  constexpr bool AHEAD = BIG && RT == 2;
+  StepPages pages = {};
+  if (AHEAD && k_begin < k_end) pages = step_pages(a, table, k_begin, t.lo, t.hi);
+  auto issue = [&](StepRegs<DT>& regs, int k) {
+    if (BIG && !AHEAD) pages = step_pages(a, table, k, t.lo, t.hi);
+    load_step<DT, BIG>(regs, a, table, pages, kvh, k, t.lo, t.hi, r, q);
+    if (AHEAD && k + 32 < k_end) pages = step_pages(a, table, k + 32, t.lo, t.hi);
+  };
 #pragma unroll
   for (int i = 0; i < PF; ++i)
-    if (k_begin + 32 * i < k_end) load_step<DT, BIG>(ring[i], a, table, kvh, k_begin + 32 * i, t.lo, t.hi, r, q);
+    if (k_begin + 32 * i < k_end) issue(ring[i], k_begin + 32 * i);
   for (int kb = k_begin; kb < k_end; kb += 32 * PF) {
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       const int k = kb + 32 * i;
       if (k < k_end) {
         compute_step(ring[i], k);
-        if (k + 32 * PF < k_end) load_step<DT, BIG>(ring[i], a, table, kvh, k + 32 * PF, t.lo, t.hi, r, q);
+        if (k + 32 * PF < k_end) issue(ring[i], k + 32 * PF);
       }
     }
   }
