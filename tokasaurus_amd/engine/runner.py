@@ -159,7 +159,8 @@ class RecordedDecodeStep:
                 gc.enable()
 
     def _forward(self):
-        logits = self.model.forward(self.ctx, self.caches, self.storage.states, self.want_rows)
+        # every row of a recorded step is wanted, in order: nothing to pick out
+        logits = self.model.forward(self.ctx, self.caches, self.storage.states, None)
         ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.token_slots, self.storage.last_token)
         return logits, ids, logprobs
 
@@ -363,7 +364,8 @@ class ModelRunner:
             hb = layout(planned, self.model.spec.vocab_size, len(self.groups))
             ctx, want_rows, tables = to_device(hb, self.model.dtype, self.model.device, self.storage.last_token)
             ctx.extras["kv_bound"] = self.kv_bound(ctx.max_kv_len)
-            logits = self.model.forward(ctx, self.cache_views(tables), self.storage.states, want_rows)
+            every_row = hb.want_rows == list(range(ctx.num_tokens))
+            logits = self.model.forward(ctx, self.cache_views(tables), self.storage.states, None if every_row else want_rows)
             out = StepOutput(logits)
             if sampling is not None and logits.shape[0] > 0:
                 # rows are in the order of the entries' wants; one slot a row

@@ -59,9 +59,10 @@ class CausalLM:
         ctx: StepContext,
         caches: list[CacheView | None],
         states: list[torch.Tensor | None],
-        want_rows: torch.Tensor,
+        want_rows: torch.Tensor | None,
     ) -> torch.Tensor:
-        """Run the batch of ``ctx`` and return logits [len(want_rows), vocab] in 32-bit."""
+        """Run the batch of ``ctx`` and return logits [len(want_rows), vocab] in 32-bit;
+        ``want_rows`` None stands for every row in order (no rows are picked out then)."""
         x = self.embedding.forward(ctx)
         order = self.spec.run_order
         last = len(order) - 1
@@ -75,6 +76,6 @@ class CausalLM:
             else:
                 out = block.forward(x, ctx, caches[i], states[i], rows)
             x, prepared = stream_and_prepared(out)
-        if last < 0:
+        if last < 0 and want_rows is not None:
             x = ops.gather_rows(x, want_rows)
         return self.head.forward(x, prepared)
