@@ -16,6 +16,7 @@ from dataclasses import dataclass, field
 
 import torch
 
+from tokasaurus_amd.kernels.upload import upload
 from tokasaurus_amd.parts.base import StepContext
 
 FROM_SLOT = None  # tokens=None: the one token is the slot's last sampled token
@@ -124,7 +125,7 @@ def to_device(hb: HostBatch, dtype: torch.dtype, device: torch.device, last_toke
     for g, table in enumerate(hb.block_tables):
         widths.append(len(table[0]) if table else 1)
         put(f"table{g}", [p for row in table for p in row])
-    packed = torch.tensor(flat, dtype=torch.int32).to(device, non_blocking=False)
+    packed = upload(flat, torch.int32, device)  # the host does not wait for the device here
 
     def view(name: str) -> torch.Tensor:
         a, m = spans[name]

@@ -21,6 +21,7 @@ from tokasaurus_amd.cache.manager import CacheManager, plan_groups
 from tokasaurus_amd.cache.storage import CacheStorage
 from tokasaurus_amd.engine.batch import PlannedEntry, StepEntry, layout, to_device
 from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.kernels.upload import upload
 from tokasaurus_amd.models.causal_lm import CausalLM
 from tokasaurus_amd.models.registry import build_model, config_from_folder
 from tokasaurus_amd.parts.base import CacheView, StepContext
@@ -371,10 +372,11 @@ class ModelRunner:
                 # rows are in the order of the entries' wants; one slot a row
                 slots = [e.slot for e in planned for _ in e.want]
                 dev = self.model.device
-                params = torch.tensor([sampling.temperatures, sampling.uniforms], dtype=torch.float32).to(dev)
-                slot_t = torch.tensor(slots, dtype=torch.int32).to(dev) if write_slots else None
+                n_out = len(sampling.temperatures)
+                params = upload(sampling.temperatures + sampling.uniforms, torch.float32, dev)
+                slot_t = upload(slots, torch.int32, dev) if write_slots else None
                 out.ids, out.logprobs = ops.sample(
-                    logits, params[0], params[1], slot_t, self.storage.last_token if write_slots else None
+                    logits, params[:n_out], params[n_out:], slot_t, self.storage.last_token if write_slots else None
                 )
         if out.ids is not None and out.ids.shape[0] > 0:
             self._copy_to_host(out)

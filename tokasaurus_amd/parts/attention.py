@@ -16,6 +16,7 @@ from dataclasses import dataclass
 import torch
 
 from tokasaurus_amd.kernels import ops
+from tokasaurus_amd.kernels.upload import upload
 from tokasaurus_amd.parts.base import (
     MIXERS,
     POSITION_ENCODINGS,
@@ -76,7 +77,7 @@ def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int) -> Att
             lists.append((req, row0, row1, 2, whole, 1))
         # one upload for all the tile lists of the step
         flat = [x for req, row0, row1, *_ in lists for x in (req + row0 + (row1 or []))]
-        dev = torch.tensor(flat, dtype=torch.int32).to(ctx.device) if flat else None
+        dev = upload(flat, torch.int32, ctx.device) if flat else None
         launches, at = [], 0
         for req, row0, row1, row_tiles, split, waves in lists:
             n = len(req)
