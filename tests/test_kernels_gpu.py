@@ -483,3 +483,28 @@ def test_kernels_refuse_what_they_cannot_do():
         ops.key_pages_shape(4, 2, 16, 20)
     with pytest.raises(KernelError, match="groups of 4"):
         ops.value_pages_shape(4, 2, 6, 64)
+
+
+def test_uploads_through_the_pinned_ring_arrive_whole():
+    """More uploads than the ring has buffers, of growing and shrinking sizes, int and float:
+    every one arrives as it was written, also while the device is busy with earlier work."""
+    from tokasaurus_amd.kernels.upload import upload
+
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(0)
+    busy = torch.randn((2048, 2048), device=dev)
+    sent, got = [], []
+    for i in range(50):
+        n = [3, 70000, 1, 0, 513][i % 5]
+        if i % 2:
+            vals = torch.randint(-(2**31), 2**31 - 1, (n,), generator=g, dtype=torch.int64).tolist()
+            dtype = torch.int32
+        else:
+            vals = torch.randn((n,), generator=g).tolist()
+            dtype = torch.float32
+        busy = busy @ busy * 1e-3  # keeps the stream occupied between uploads
+        sent.append(torch.tensor(vals, dtype=dtype))
+        got.append(upload(vals, dtype, dev))
+    torch.cuda.synchronize()
+    for a, b in zip(sent, got):
+        assert b.dtype == a.dtype and torch.equal(b.cpu(), a)
