@@ -113,3 +113,13 @@ def test_finalize_derives_and_checks():
         EngineConfig(kv_cache_num_tokens=100, page_size=16).finalize()
     with pytest.raises(OptionError, match="dtype"):
         EngineConfig(dtype="float16").finalize()
+
+
+def test_settings_of_the_reference_that_are_not_built_are_refused():
+    from tokasaurus_amd.config.engine_config import EngineConfig, OptionError
+
+    for kw, msg in ((dict(greedy_prefill=False), "paced prefill"), (dict(max_topk_logprobs=5), "not offered"),
+                    (dict(log_level="chatty"), "logging level"), (dict(scheduling_steps_ahead=-1), "negative")):
+        with pytest.raises(OptionError, match=msg):
+            EngineConfig(kv_cache_num_tokens=1024, **kw).finalize()
+    EngineConfig(kv_cache_num_tokens=1024, scheduling_steps_ahead=0, log_level="debug").finalize()

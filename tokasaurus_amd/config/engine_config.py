@@ -35,8 +35,8 @@ class EngineConfig:
     max_tokens_per_forward: int = 8192
     max_seqs_per_forward: int = 1024
     max_num_tokens_per_request: int | None = None
-    prefill_round_up_multiple: int = 16
-    greedy_prefill: bool = True
+    prefill_round_up_multiple: int = 16  # rounds the paced prefill of the reference; without effect on the greedy one
+    greedy_prefill: bool = True  # the reference's default is F (paced prefill), which is not built here
 
     # --- outputs (tokasaurus/common_types.py:64-65)
     enable_chosen_logprobs: bool = True
@@ -82,6 +82,14 @@ class EngineConfig:
                 raise OptionError(f"{name} must be positive")
         if self.scheduling_steps_ahead < 0:
             raise OptionError("scheduling_steps_ahead must not be negative")
+        # options of the reference whose other settings this engine does not build: say so
+        # instead of going on as if they had been honoured
+        if not self.greedy_prefill:
+            raise OptionError("greedy_prefill=F (the reference's paced prefill) is not built: prompts take what the token budget leaves")
+        if self.max_topk_logprobs is not None:
+            raise OptionError("max_topk_logprobs is not offered: only the chosen token's log-probability is returned")
+        if self.log_level.upper() not in ("DEBUG", "INFO", "WARNING", "ERROR", "CRITICAL"):
+            raise OptionError(f"log_level {self.log_level!r} is no logging level")
         self.kv_cache_num_blocks()
         if self.max_num_tokens_per_request is None and max_position_embeddings is not None:
             self.max_num_tokens_per_request = min(max_position_embeddings, self.kv_cache_num_tokens)

@@ -13,6 +13,7 @@ it to the request's slot and the next step's embedding reads it from there
 
 from __future__ import annotations
 
+import logging
 import time
 from dataclasses import dataclass, field
 
@@ -23,6 +24,9 @@ from tokasaurus_amd.engine.batch import StepEntry
 from tokasaurus_amd.engine.runner import ModelRunner, Sampling, StepOutput
 from tokasaurus_amd.engine.scheduler import Decision, Request, Scheduler
 from tokasaurus_amd.sampling import SamplingParams, uniform_for
+
+
+log = logging.getLogger("tokasaurus_amd")
 
 
 @dataclass
@@ -68,6 +72,9 @@ class Engine:
         if config.model is None and runner is None:
             raise ValueError("EngineConfig.model is not set")
         self.config = config
+        if not log.handlers and not logging.getLogger().handlers:
+            logging.basicConfig(format="%(asctime)s %(name)s %(levelname)s %(message)s")
+        log.setLevel(config.log_level.upper())
         if runner is None:
             from tokasaurus_amd.models.registry import config_from_folder
 
@@ -192,9 +199,15 @@ class Engine:
         return done
 
     def run_until_done(self) -> list[Completion]:
+        """Step until nothing is left; every ``stats_report_seconds`` a line of counters goes to
+        the log (the reference's stats line, tokasaurus/manager/monitoring.py:179-232)."""
         done: list[Completion] = []
+        last = time.perf_counter()
         while self.has_work():
             done.extend(self.step())
+            if self.config.stats_report_seconds > 0 and time.perf_counter() - last >= self.config.stats_report_seconds:
+                last = time.perf_counter()
+                log.info("stats %s", {k: (round(v, 1) if isinstance(v, float) else v) for k, v in self.stats.as_dict().items()})
         return done
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams] | None = None) -> list[Completion]:
