@@ -242,9 +242,16 @@ class ModelRunner:
             self.groups, num_pages, page_size, max_slots, max_blocks_per_request=-(-limit // page_size)
         )
         self.use_graphs = use_graphs
-        self.graph_sizes = [b for b in graph_buckets(graph_max_size, graph_step) if b <= max(max_slots, 1)] if use_graphs else []
-        if use_graphs and max_slots < graph_max_size and max_slots not in self.graph_sizes:
-            self.graph_sizes.append(max_slots)
+        # Only this engine's own kernels go into a recording.  In bfloat16, steps of more rows
+        # than the weight-streaming product takes on hold library products, which may keep
+        # work memory that they clear in ways a replay does not repeat: such steps run eagerly
+        # (the step launched ahead hides their launches; measured 1 to 2 % slower at 40 and 64 rows).
+        if model.dtype == torch.bfloat16:
+            graph_max_size = min(graph_max_size, ops.SKINNY_ROWS)
+        largest = min(graph_max_size, max(max_slots, 1))
+        self.graph_sizes = [b for b in graph_buckets(graph_max_size, graph_step) if b <= largest] if use_graphs else []
+        if use_graphs and largest not in self.graph_sizes:
+            self.graph_sizes.append(largest)
             self.graph_sizes.sort()
         self.recorded: dict[tuple[int, int], RecordedDecodeStep] = {}  # by (rows, context bound)
         self.graph_pool = torch.cuda.graph_pool_handle() if use_graphs else None
