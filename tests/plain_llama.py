@@ -264,6 +264,15 @@ def sample(logits: torch.Tensor, temperature: float, u: float) -> tuple[int, flo
     return token, float(torch.log(probs[token]))
 
 
+def topk_logprobs(logits: torch.Tensor, temperature: float, k: int) -> tuple[list[int], list[float]]:
+    """llama.py:407-412 for one row: the k largest probabilities of softmax(logits / T)
+    and their logarithms, largest first (T 0 counts as 1, model/types.py:302-312)."""
+    divisor = temperature if temperature > 0 else 1.0
+    probs = torch.softmax(logits.to(torch.float32) / divisor, dim=-1)
+    top, ids = torch.topk(probs, k=k, dim=-1)
+    return ids.tolist(), top.log().tolist()
+
+
 def greedy_generate(
     cfg: dict, w: dict[str, torch.Tensor], prompt: list[int], max_tokens: int
 ) -> list[int]:

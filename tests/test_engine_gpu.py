@@ -76,6 +76,41 @@ def test_temperature_generation_config_b_in_portions_of_16(folders):
     assert engine.stats.steps > 130 // 16
 
 
+@pytest.mark.parametrize("graphs", [True, False])
+def test_ranked_tokens_and_their_logprobs(folders, graphs):
+    """max_topk_logprobs=4: a request that asks for 3 gets every token's 3 most probable
+    tokens, one that asks for none gets none, one that asks for more than 4 is refused."""
+    cfg, _ = TINY["B"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 30 + n) for n in (9, 40, 3)]
+    engine = engine_for(folders, "B", max_topk_logprobs=4, max_prefill_chunk=16, seed=2, use_hipgraphs=graphs)
+    params = [SamplingParams(temperature=0.7, max_tokens=6, ignore_eos=True, seed=7, topk_logprobs=3),
+              SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, topk_logprobs=4),
+              SamplingParams(temperature=0.7, max_tokens=6, ignore_eos=True, seed=9)]
+    with pytest.raises(ValueError, match="max_topk_logprobs=4"):
+        engine.submit(prompts[0], SamplingParams(topk_logprobs=5))
+    done = engine.generate(prompts, params)
+    assert done[2].topk_ids is None and len(done[2].tokens) == 6
+    pcfg, w = plain_llama.load_folder(folders["B"])
+    for c, p, prompt in zip(done[:2], params[:2], prompts[:2]):
+        want, _ = plain_generate(folders["B"], prompt, 6, temperature=p.temperature, engine_seed=2, request_seed=p.seed or 0)
+        if p.temperature > 0:
+            assert c.tokens == want
+        assert len(c.topk_ids) == len(c.topk_logprobs) == 6
+        ids = list(prompt)
+        for tok, lp, top_ids, top_lps in zip(c.tokens, c.logprobs, c.topk_ids, c.topk_logprobs):
+            logits = plain_llama.forward_logits(pcfg, w, ids)[-1]
+            want_ids, want_lps = plain_llama.topk_logprobs(logits, p.temperature, p.topk_logprobs)
+            assert top_ids == want_ids
+            assert torch.allclose(torch.tensor(top_lps), torch.tensor(want_lps), atol=1e-4)
+            if p.temperature == 0:
+                assert top_ids[0] == tok and abs(top_lps[0] - lp) < 1e-5
+            elif tok in top_ids:
+                assert abs(top_lps[top_ids.index(tok)] - lp) < 1e-5
+            ids.append(tok)
+    if graphs:
+        assert engine.runner.recorded
+
+
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_bfloat16_generation_follows_the_plain_one(folders, name):
     cfg, _ = TINY[name]

@@ -146,6 +146,59 @@ def test_sample_frequencies_follow_the_probabilities():
     assert float((freq - probs).abs().max()) < 0.03
 
 
+@pytest.mark.parametrize("vocab, k", [(333, 1), (1000, 5), (2049, 32), (128256, 5), (128256, 20), (40, 32)])
+def test_topk_logprobs(vocab, k):
+    import plain_llama
+    from tokasaurus_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(vocab + k)
+    rows = 7
+    logits = torch.randn((rows, vocab), generator=g) * 3.0
+    # the best tokens of row 2 lie in one chunk and at the vocabulary's end; row 4 holds ties
+    logits[2, -min(k, vocab):] += 20.0
+    logits[4, 3] = logits[4, vocab // 2] = logits[4, vocab - 1] = logits[4].max() + 1.0
+    temps = [0.0, 0.8, 1.0, 0.3, 2.0, 0.8, 1e-2]
+    ids, lps = ops.topk_logprobs(logits.cuda(), torch.tensor(temps).cuda(), k)
+    assert ids.shape == (rows, k) and lps.shape == (rows, k)
+    ids, lps = ids.cpu(), lps.cpu()
+    for r in range(rows):
+        T = temps[r] if temps[r] > 0 else 1.0
+        ref = torch.log_softmax(logits[r].double() / T, -1)
+        want_ids, want_lps = plain_llama.topk_logprobs(logits[r], temps[r], k)
+        got = ids[r].tolist()
+        assert len(set(got)) == k and all(0 <= t < vocab for t in got)
+        # each place holds the log-probability of its own token, and the places descend
+        for j, t in enumerate(got):
+            assert abs(float(lps[r, j]) - float(ref[t])) < 1e-3 + 1e-4 * abs(float(ref[t])), (r, j)
+        order = [(-float(logits[r, t]), t) for t in got]
+        assert order == sorted(order), (r, got)
+        # the same tokens as the plain ranking (random logits of distinct values), as far as the
+        # plain one can tell them apart: it ranks probabilities, which a small temperature
+        # rounds to zero, where the kernel ranks the logits themselves
+        if r != 4:
+            seen = [j for j in range(k) if want_lps[j] > -80.0]
+            assert [got[j] for j in seen] == [want_ids[j] for j in seen], (r, got, want_ids)
+        # nothing outside the list beats its last place
+        rest = logits[r].clone()
+        rest[got] = -float("inf")
+        assert float(rest.max()) <= float(logits[r, got[-1]])
+    if k >= 3:
+        assert ids[4, :3].tolist() == [3, vocab // 2, vocab - 1]  # equal logits: the lower index first
+
+
+def test_topk_logprobs_refusals():
+    from tokasaurus_amd.kernels import ops
+    from tokasaurus_amd.kernels.library import KernelError
+
+    logits = torch.zeros((2, 50), device="cuda")
+    temps = torch.ones((2,), device="cuda")
+    for k in (0, 33, 51):
+        with pytest.raises((KernelError, ValueError)):
+            ops.topk_logprobs(logits, temps, k)
+    ids, lps = ops.topk_logprobs(logits[:0], temps[:0], 3)
+    assert ids.shape == (0, 3)
+
+
 # --------------------------------------------------------------------------
 # matrix products
 # --------------------------------------------------------------------------

@@ -251,6 +251,21 @@ def test_layer_order_and_folder_loading(tmp_path):
 # ---- sampling --------------------------------------------------------------
 
 
+def test_topk_logprobs():
+    logits = torch.tensor([0.1, 2.0, -1.0, 3.0, 0.5])
+    ids, lps = pl.topk_logprobs(logits, 0.5, 3)
+    assert ids == [3, 1, 4]
+    want = torch.log_softmax(logits / 0.5, -1)
+    assert torch.allclose(torch.tensor(lps), want[[3, 1, 4]], atol=1e-6)
+    # the first place is the greedy token with the log-probability the sampler reports for it
+    tok, lp = pl.sample(logits, 0.0, 0.0)
+    ids, lps = pl.topk_logprobs(logits, 0.0, 1)
+    assert ids == [tok] and abs(lps[0] - lp) < 1e-6
+    # all of them: the probabilities sum to one
+    _, lps = pl.topk_logprobs(logits, 1.3, 5)
+    assert abs(sum(math.exp(x) for x in lps) - 1.0) < 1e-5
+
+
 def test_sampling():
     logits = torch.tensor([0.1, 2.0, -1.0, 2.0, 0.5])
     tok, lp = pl.sample(logits, 0.0, 0.3)

@@ -273,3 +273,17 @@ def test_an_end_token_found_a_step_late_costs_one_token_and_no_more():
     assert [r.id for r in done] == ["a"] and done[0].completion == [3] and done[0].finish_reason == "stop"
     assert cache.num_free_pages() == [64] and not s.has_work()
     assert s.resolve(d1, [7], [0.0]) == [] and done[0].completion == [3]  # dropped
+
+
+def test_ranked_tokens_are_kept_only_as_far_as_a_request_asked():
+    s, _ = make()
+    s.submit(req("a", 3, 2, topk_logprobs=2))
+    s.submit(req("b", 3, 2))
+    for step in range(2):
+        d = s.schedule(); s.advance(d)
+        rows = len(d.outputs)
+        topk = ([[10 * step + i, 50, 60] for i in range(rows)], [[-0.1, -1.0, -2.0]] * rows)
+        done = s.resolve(d, [7] * rows, [0.0] * rows, topk)
+    by_id = {r.id: r for r in done}
+    assert by_id["a"].topk_ids == [[0, 50], [10, 50]] and by_id["a"].topk_logprobs == [[-0.1, -1.0]] * 2
+    assert by_id["b"].topk_ids == [] and by_id["b"].completion == [7, 7]

@@ -22,6 +22,9 @@ class OptionError(ValueError):
     """A command-line argument the engine cannot accept."""
 
 
+MAX_TOPK_LOGPROBS = 32  # the most tokens the ranking kernel orders for a row
+
+
 @dataclass
 class EngineConfig:
     # --- model (tokasaurus/common_types.py:53-58)
@@ -40,7 +43,7 @@ class EngineConfig:
 
     # --- outputs (tokasaurus/common_types.py:64-65)
     enable_chosen_logprobs: bool = True
-    max_topk_logprobs: int | None = None
+    max_topk_logprobs: int | None = None  # when set, every step ranks this many tokens; requests ask for up to as many
 
     # --- launch-overhead removal (tokasaurus/common_types.py:117-121); here HIP graphs
     use_hipgraphs: bool = True
@@ -86,8 +89,8 @@ class EngineConfig:
         # instead of going on as if they had been honoured
         if not self.greedy_prefill:
             raise OptionError("greedy_prefill=F (the reference's paced prefill) is not built: prompts take what the token budget leaves")
-        if self.max_topk_logprobs is not None:
-            raise OptionError("max_topk_logprobs is not offered: only the chosen token's log-probability is returned")
+        if self.max_topk_logprobs is not None and not 1 <= self.max_topk_logprobs <= MAX_TOPK_LOGPROBS:
+            raise OptionError(f"max_topk_logprobs must be between 1 and {MAX_TOPK_LOGPROBS} (what the ranking kernel takes)")
         if self.log_level.upper() not in ("DEBUG", "INFO", "WARNING", "ERROR", "CRITICAL"):
             raise OptionError(f"log_level {self.log_level!r} is no logging level")
         self.kv_cache_num_blocks()

@@ -195,3 +195,147 @@ TK_API int tk_sample(const float* logits, int ld, int rows, int vocab, const flo
   TK_CHECK_LAUNCH("sample_finish");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// The k most probable tokens of every row and their log-probabilities under
+// softmax(logits / T) (T treated as 1 when 0), most probable first; among equal
+// logits the lower index first.  Two kernels, cut like the sampler's:
+//   topk_partial: one workgroup per (row, chunk): the chunk's k best in order, its
+//                 maximum and sum exp((x - max) / T);
+//   topk_finish:  one workgroup per row: the k best among the chunks' candidates.
+// Each of the k places is one arg-max over what comes after the place before it in
+// the order (value descending, index ascending): k is small, the candidates are few.
+#define TOPK_MAX 32
+
+struct Ranked {
+  float v;
+  int i;
+};
+
+// a stands before b in the order of the result
+__device__ __forceinline__ bool before(const Ranked& a, const Ranked& b) {
+  return a.v > b.v || (a.v == b.v && a.i < b.i);
+}
+
+// what is left when nothing more is eligible: it stands behind every real element
+__device__ __forceinline__ Ranked nothing() { return Ranked{-INFINITY, 0x7fffffff}; }
+
+// the first in the order over the workgroup; every thread gets it
+__device__ __forceinline__ Ranked block_first(Ranked mine, Ranked* red) {
+  const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
+#pragma unroll
+  for (int o = TK_WAVE / 2; o > 0; o >>= 1) {
+    Ranked other{__shfl_xor(mine.v, o, TK_WAVE), __shfl_xor(mine.i, o, TK_WAVE)};
+    if (before(other, mine)) mine = other;
+  }
+  __syncthreads();  // the round before has read red
+  if (lane == 0) red[wave] = mine;
+  __syncthreads();
+  Ranked best = red[0];
+  for (int w = 1; w < SM_THREADS / TK_WAVE; ++w)
+    if (before(red[w], best)) best = red[w];
+  return best;
+}
+
+__global__ __launch_bounds__(SM_THREADS) void topk_partial_kernel(
+    const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ temperature, int k,
+    float* __restrict__ part_val, int* __restrict__ part_idx, float* __restrict__ part_max,
+    float* __restrict__ part_sum, int n_chunks) {
+  __shared__ Ranked red[SM_THREADS / TK_WAVE];
+  __shared__ float red_f[16];
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const float* x = logits + (size_t)row * ld;
+  const float T = temperature[row];
+  const float inv_t = T > 0.f ? 1.0f / T : 1.0f;
+  const int begin = chunk * SM_CHUNK + tid * SM_PER_THREAD;
+  Ranked held[SM_PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < SM_PER_THREAD; ++i)
+    held[i] = begin + i < vocab ? Ranked{x[begin + i], begin + i} : nothing();
+  const size_t o = (size_t)row * n_chunks + chunk;
+  Ranked prev{INFINITY, -1};
+  float chunk_max = -INFINITY;
+  for (int r = 0; r < k; ++r) {
+    Ranked mine = nothing();
+#pragma unroll
+    for (int i = 0; i < SM_PER_THREAD; ++i)
+      if (before(prev, held[i]) && before(held[i], mine)) mine = held[i];
+    prev = block_first(mine, red);
+    if (r == 0) chunk_max = prev.v;
+    if (tid == 0) {
+      part_val[o * k + r] = prev.v;
+      part_idx[o * k + r] = prev.i;
+    }
+  }
+  float local = 0.f;
+#pragma unroll
+  for (int i = 0; i < SM_PER_THREAD; ++i)
+    local += (held[i].v == -INFINITY) ? 0.f : expf((held[i].v - chunk_max) * inv_t);
+  const float total = block_sum(local, red_f);
+  if (tid == 0) {
+    part_max[o] = chunk_max;
+    part_sum[o] = total;
+  }
+}
+
+__global__ __launch_bounds__(SM_THREADS) void topk_finish_kernel(
+    const float* __restrict__ temperature, int k, const float* __restrict__ part_val,
+    const int* __restrict__ part_idx, const float* __restrict__ part_max,
+    const float* __restrict__ part_sum, int n_chunks, int* __restrict__ out_ids,
+    float* __restrict__ out_logprobs) {
+  __shared__ Ranked red[SM_THREADS / TK_WAVE];
+  __shared__ float red_f[16];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float T = temperature[row];
+  const float inv_t = T > 0.f ? 1.0f / T : 1.0f;
+  const float* pm = part_max + (size_t)row * n_chunks;
+  const float* ps = part_sum + (size_t)row * n_chunks;
+  const float* pv = part_val + (size_t)row * n_chunks * k;
+  const int* pi = part_idx + (size_t)row * n_chunks * k;
+  const int n = n_chunks * k;
+  float m = -INFINITY;
+  for (int c = tid; c < n_chunks; c += SM_THREADS) m = fmaxf(m, pm[c]);
+  const float row_max = block_max(m, red_f);
+  float mass = 0.f;
+  for (int c = tid; c < n_chunks; c += SM_THREADS)
+    mass += (pm[c] == -INFINITY) ? 0.f : ps[c] * expf((pm[c] - row_max) * inv_t);
+  const float log_total = logf(block_sum(mass, red_f));
+  Ranked prev{INFINITY, -1};
+  for (int r = 0; r < k; ++r) {
+    Ranked mine = nothing();
+    for (int c = tid; c < n; c += SM_THREADS) {
+      const Ranked cand{pv[c], pi[c]};
+      if (before(prev, cand) && before(cand, mine)) mine = cand;
+    }
+    prev = block_first(mine, red);
+    if (tid == 0) {
+      out_ids[(size_t)row * k + r] = prev.i;
+      out_logprobs[(size_t)row * k + r] = (prev.v - row_max) * inv_t - log_total;
+    }
+  }
+}
+
+// part_val and part_idx hold rows * tk_sample_chunks(vocab) * k entries, part_max and part_sum
+// rows * tk_sample_chunks(vocab); out_ids and out_logprobs are [rows, k].
+TK_API int tk_topk_logprobs(const float* logits, int ld, int rows, int vocab, const float* temperature,
+                            int k, int* out_ids, float* out_logprobs, float* part_val, int* part_idx,
+                            float* part_max, float* part_sum, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "topk_logprobs: bad sizes rows=%d vocab=%d ld=%d",
+             rows, vocab, ld);
+  TK_REQUIRE(k >= 1 && k <= TOPK_MAX && k <= vocab,
+             "topk_logprobs: k=%d is not between 1 and %d (and at most the vocabulary of %d)", k,
+             TOPK_MAX, vocab);
+  const int n_chunks = (vocab + SM_CHUNK - 1) / SM_CHUNK;
+  TK_REQUIRE(n_chunks <= SM_MAX_CHUNKS, "topk_logprobs: a vocabulary of %d is larger than %d", vocab,
+             SM_MAX_CHUNKS * SM_CHUNK);
+  TK_REQUIRE(rows < 65536, "topk_logprobs: %d rows are too many for one call", rows);
+  TK_REQUIRE(part_val && part_idx && part_max && part_sum, "topk_logprobs: scratch missing");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(topk_partial_kernel, dim3(n_chunks, rows), dim3(SM_THREADS), 0, stream, logits,
+                     ld, vocab, temperature, k, part_val, part_idx, part_max, part_sum, n_chunks);
+  TK_CHECK_LAUNCH("topk_partial");
+  hipLaunchKernelGGL(topk_finish_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, temperature, k,
+                     part_val, part_idx, part_max, part_sum, n_chunks, out_ids, out_logprobs);
+  TK_CHECK_LAUNCH("topk_finish");
+  return 0;
+}

@@ -37,6 +37,9 @@ class Completion:
     logprobs: list[float]
     finish_reason: str
     times_bumped: int = 0
+    # for a request that asked for them: every token's most probable alternatives, most probable first
+    topk_ids: list[list[int]] | None = None
+    topk_logprobs: list[list[float]] | None = None
 
 
 @dataclass
@@ -91,6 +94,7 @@ class Engine:
                 use_graphs=config.use_hipgraphs,
                 graph_max_size=config.hipgraph_max_size,
                 graph_step=config.hipgraph_step,
+                topk_logprobs=config.max_topk_logprobs,
             )
         else:
             config.finalize(runner.max_positions)
@@ -114,6 +118,10 @@ class Engine:
     # ---- requests
     def submit(self, prompt: list[int], params: SamplingParams | None = None, request_id: str | None = None) -> str:
         params = params or SamplingParams()
+        if params.topk_logprobs is not None and params.topk_logprobs > (self.config.max_topk_logprobs or 0):
+            # tokasaurus/server/utils.py:449-456
+            raise ValueError(f"topk_logprobs={params.topk_logprobs} but the engine was configured with "
+                             f"max_topk_logprobs={self.config.max_topk_logprobs}")
         if request_id is None:
             request_id = f"req-{self._next_id}"
         vocab = self.runner.model.spec.vocab_size
@@ -169,11 +177,14 @@ class Engine:
         decision, out = launched
         tokens, logprobs = out.sampled()
         keep_logprobs = self.config.enable_chosen_logprobs and out.logprobs is not None
-        finished = self.scheduler.resolve(decision, tokens, logprobs if keep_logprobs else None)
+        finished = self.scheduler.resolve(decision, tokens, logprobs if keep_logprobs else None, out.topk())
         done = []
         for r in finished:
             self._request_seed.pop(r.id, None)
-            done.append(Completion(r.id, r.prompt, list(r.completion), list(r.logprobs), r.finish_reason or "", r.times_bumped))
+            c = Completion(r.id, r.prompt, list(r.completion), list(r.logprobs), r.finish_reason or "", r.times_bumped)
+            if r.params.topk_logprobs:
+                c.topk_ids, c.topk_logprobs = list(r.topk_ids), list(r.topk_logprobs)
+            done.append(c)
         return done
 
     def step(self) -> list[Completion]:

@@ -31,6 +31,7 @@ class RunConfig(EngineConfig):
     max_tokens: int = 16
     temperature: float = 0.0
     ignore_eos: bool = False
+    topk_logprobs: int | None = None  # per token, this many most probable tokens (needs max_topk_logprobs)
 
 
 def prepare_model_folder(config: RunConfig) -> None:
@@ -79,9 +80,13 @@ def start(config: RunConfig) -> int:
     else:
         g = torch.Generator().manual_seed(config.seed)
         prompts = [torch.randint(0, vocab, (config.prompt_len,), generator=g).tolist() for _ in range(config.num_prompts)]
-    params = SamplingParams(temperature=config.temperature, max_tokens=config.max_tokens, ignore_eos=config.ignore_eos)
+    params = SamplingParams(temperature=config.temperature, max_tokens=config.max_tokens, ignore_eos=config.ignore_eos,
+                            topk_logprobs=config.topk_logprobs)
     for c in engine.generate(prompts, params):
-        print(json.dumps({"id": c.request_id, "tokens": c.tokens, "logprobs": c.logprobs, "finish_reason": c.finish_reason}))
+        line = {"id": c.request_id, "tokens": c.tokens, "logprobs": c.logprobs, "finish_reason": c.finish_reason}
+        if c.topk_ids is not None:
+            line["topk_ids"], line["topk_logprobs"] = c.topk_ids, c.topk_logprobs
+        print(json.dumps(line))
     print(json.dumps({"stats": engine.stats.as_dict()}), file=sys.stderr)
     return 0
 

@@ -49,9 +49,11 @@ class StepOutput:
     logits: torch.Tensor  # [wanted, vocab] float32
     ids: torch.Tensor | None = None  # [wanted] int32, when the step sampled
     logprobs: torch.Tensor | None = None
+    topk_ids: torch.Tensor | None = None  # [wanted, k] int32, when the runner ranks the most probable tokens
+    topk_logprobs: torch.Tensor | None = None  # [wanted, k] float32
     # a sampled step also copies ids and log-probabilities to pinned host memory, in stream
     # order right behind the step: they can be read while later steps already run
-    host: torch.Tensor | None = None  # [2, >= wanted] int32 (row 1 holds the bits of float32)
+    host: "HostResults | None" = None
     ready: torch.cuda.Event | None = None
 
     def sampled(self) -> tuple[list[int], list[float]]:
@@ -62,7 +64,33 @@ class StepOutput:
         if self.host is None:
             return self.ids.tolist(), (self.logprobs.tolist() if self.logprobs is not None else [])
         self.ready.synchronize()
-        return self.host[0, :n].tolist(), self.host[1, :n].view(torch.float32).tolist()
+        return self.host.ids[:n].tolist(), self.host.logprobs[:n].tolist()
+
+    def topk(self) -> tuple[list[list[int]], list[list[float]]] | None:
+        """For every sampled row the most probable tokens and their log-probabilities, most
+        probable first; None when the runner ranks none."""
+        if self.topk_ids is None:
+            return None
+        n, k = self.topk_ids.shape
+        if self.host is None:
+            return self.topk_ids.tolist(), self.topk_logprobs.tolist()
+        self.ready.synchronize()
+        return (self.host.topk_ids[: n * k].view(n, k).tolist(),
+                self.host.topk_logprobs[: n * k].view(n, k).tolist())
+
+
+class HostResults:
+    """Pinned host memory for one step's sampled ids, log-probabilities and ranked tokens:
+    one allocation, viewed by kind."""
+
+    def __init__(self, width: int, k: int):
+        self.width, self.k = width, k
+        self.buffer = torch.zeros((width * (2 + 2 * k),), dtype=torch.int32, pin_memory=True)
+        self.ids = self.buffer[:width]
+        self.logprobs = self.buffer[width : 2 * width].view(torch.float32)
+        self.topk_ids = self.buffer[2 * width : (2 + k) * width]
+        self.topk_logprobs = self.buffer[(2 + k) * width :].view(torch.float32)
+        self.event = torch.cuda.Event()
 
 
 def graph_buckets(max_size: int, step: int) -> list[int]:
@@ -95,6 +123,7 @@ class RecordedDecodeStep:
         # cycle, or they would be freed by the cyclic collector at a time of its choosing,
         # possibly while another step is being recorded, when memory must not be released
         self.size = size
+        self.num_ranked = runner.topk_logprobs
         model, storage, manager = runner.model, runner.storage, runner.manager
         self.model, self.storage, self.manager = model, storage, manager
         device = model.device
@@ -153,7 +182,7 @@ class RecordedDecodeStep:
             # recorded steps run one at a time and their results are read before the next step:
             # they share one pool of memory
             with torch.cuda.graph(self.graph, pool=runner.graph_pool):
-                self.logits, self.ids, self.logprobs = self._forward()
+                self.logits, self.ids, self.logprobs, self.topk = self._forward()
             torch.cuda.synchronize()
         finally:
             if was_enabled:
@@ -163,7 +192,8 @@ class RecordedDecodeStep:
         # every row of a recorded step is wanted, in order: nothing to pick out
         logits = self.model.forward(self.ctx, self.caches, self.storage.states, None)
         ids, logprobs = ops.sample(logits, self.temperature, self.uniform, self.token_slots, self.storage.last_token)
-        return logits, ids, logprobs
+        topk = ops.topk_logprobs(logits, self.temperature, self.num_ranked) if self.num_ranked else None
+        return logits, ids, logprobs, topk
 
     def _fill(self, token_ids, positions, slots, write_slots, temperatures, uniforms) -> None:
         B, n = self.size, len(token_ids)
@@ -212,7 +242,10 @@ class RecordedDecodeStep:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
         self.graph.replay()
-        return StepOutput(self.logits[:n], self.ids[:n], self.logprobs[:n] if self.logprobs is not None else None)
+        out = StepOutput(self.logits[:n], self.ids[:n], self.logprobs[:n] if self.logprobs is not None else None)
+        if self.topk is not None:
+            out.topk_ids, out.topk_logprobs = self.topk[0][:n], self.topk[1][:n]
+        return out
 
 
 class ModelRunner:
@@ -226,9 +259,13 @@ class ModelRunner:
         use_graphs: bool = True,
         graph_max_size: int = 128,
         graph_step: int = 16,
+        topk_logprobs: int | None = None,
     ):
         assert model.device is not None, "load the model's weights first"
         self.model = model
+        # every sampled row also gets its most probable tokens ranked, this many of them
+        # (tokasaurus/model/llama.py:407-416 ranks for every row what the engine was set up for)
+        self.topk_logprobs = int(topk_logprobs) if topk_logprobs else 0
         self.page_size = page_size
         self.max_positions = model.spec.max_positions
         limit = min(self.max_positions, num_pages * page_size)
@@ -255,7 +292,7 @@ class ModelRunner:
             self.graph_sizes.sort()
         self.recorded: dict[tuple[int, int], RecordedDecodeStep] = {}  # by (rows, context bound)
         self.graph_pool = torch.cuda.graph_pool_handle() if use_graphs else None
-        self._host_ring: list[tuple[torch.Tensor, torch.cuda.Event]] = []  # pinned buffers for sampled ids
+        self._host_ring: list[HostResults] = []  # pinned buffers for what steps sampled
         self._host_at = 0
         self.storage = CacheStorage(
             self.groups,
@@ -385,6 +422,8 @@ class ModelRunner:
                 out.ids, out.logprobs = ops.sample(
                     logits, params[:n_out], params[n_out:], slot_t, self.storage.last_token if write_slots else None
                 )
+                if self.topk_logprobs:
+                    out.topk_ids, out.topk_logprobs = ops.topk_logprobs(logits, params[:n_out], self.topk_logprobs)
         if out.ids is not None and out.ids.shape[0] > 0:
             self._copy_to_host(out)
         for e in planned:
@@ -393,18 +432,21 @@ class ModelRunner:
 
     def _copy_to_host(self, out: StepOutput) -> None:
         n = out.ids.shape[0]
-        if not self._host_ring or self._host_ring[0][0].shape[1] < n:
+        k = self.topk_logprobs
+        if not self._host_ring or self._host_ring[0].width < n:
             width = max(n, self.manager.slots.num_slots)
-            self._host_ring = [(torch.zeros((2, width), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
-                               for _ in range(4)]
-        buf, event = self._host_ring[self._host_at % len(self._host_ring)]
+            self._host_ring = [HostResults(width, k) for _ in range(4)]
+        host = self._host_ring[self._host_at % len(self._host_ring)]
         self._host_at += 1
-        event.synchronize()  # whoever used this buffer four steps ago has long read it
-        buf[0, :n].copy_(out.ids, non_blocking=True)
+        host.event.synchronize()  # whoever used this buffer four steps ago has long read it
+        host.ids[:n].copy_(out.ids, non_blocking=True)
         if out.logprobs is not None:
-            buf[1, :n].view(torch.float32).copy_(out.logprobs, non_blocking=True)
-        event.record()
-        out.host, out.ready = buf, event
+            host.logprobs[:n].copy_(out.logprobs, non_blocking=True)
+        if out.topk_ids is not None:
+            host.topk_ids[: n * k].copy_(out.topk_ids.reshape(-1), non_blocking=True)
+            host.topk_logprobs[: n * k].copy_(out.topk_logprobs.reshape(-1), non_blocking=True)
+        host.event.record()
+        out.host, out.ready = host, host.event
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         """Run one batch and return its logits only (nothing is sampled or written to slots)."""

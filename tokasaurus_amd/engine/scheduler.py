@@ -43,6 +43,8 @@ class Request:
     prompt_done: int = 0  # prompt tokens already in the cache
     completion: list[int] = field(default_factory=list)
     logprobs: list[float] = field(default_factory=list)
+    topk_ids: list[list[int]] = field(default_factory=list)  # for requests that ask for ranked tokens
+    topk_logprobs: list[list[float]] = field(default_factory=list)
     finish_reason: str | None = None
     times_bumped: int = 0
     sampled: int = 0  # completion tokens sampled so far, those whose ids have not come back included
@@ -189,6 +191,8 @@ class Scheduler:
         req.state, req.prompt_done = QUEUED, 0
         req.completion.clear()
         req.logprobs.clear()
+        req.topk_ids.clear()
+        req.topk_logprobs.clear()
         req.sampled = 0
         req.epoch += 1
         req.times_bumped += 1
@@ -246,11 +250,18 @@ class Scheduler:
         if self.sanity_checks:
             self.cache.check()
 
-    def resolve(self, decision: Decision, tokens: list[int], logprobs: list[float] | None = None) -> list[Request]:
+    def resolve(
+        self,
+        decision: Decision,
+        tokens: list[int],
+        logprobs: list[float] | None = None,
+        topk: tuple[list[list[int]], list[list[float]]] | None = None,
+    ) -> list[Request]:
         """Take the sampled tokens of an advanced step, in the order of its requests with
         output.  A token for a request that has meanwhile started again, was aborted or
-        stopped at an end token is dropped (it was computed for nothing).  Returns the
-        requests that are finished and have all their tokens."""
+        stopped at an end token is dropped (it was computed for nothing).  ``topk`` holds
+        every row's ranked tokens and their log-probabilities; a request keeps as many of
+        them as it asked for.  Returns the requests that are finished and have all their tokens."""
         assert len(tokens) == len(decision.outputs), (len(tokens), len(decision.outputs))
         finished = []
         for i, (req, epoch) in enumerate(decision.outputs):
@@ -259,6 +270,9 @@ class Scheduler:
             req.completion.append(int(tokens[i]))
             if logprobs is not None:
                 req.logprobs.append(float(logprobs[i]))
+            if topk is not None and req.params.topk_logprobs:
+                req.topk_ids.append(list(topk[0][i][: req.params.topk_logprobs]))
+                req.topk_logprobs.append(list(topk[1][i][: req.params.topk_logprobs]))
             if not req.params.ignore_eos and int(tokens[i]) in self.eos_token_ids:  # manager.py:205-206
                 if req.state != FINISHED:
                     self.decoding.pop(req.id)

@@ -37,6 +37,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
         "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_chunks": [c_int],
+        "tk_topk_logprobs": [_P, c_int, c_int, c_int, _P, c_int, _P, _P, _P, _P, _P, _P, _P],
     },
     "mfma": {
         "tk_paged_attention_mfma": [_P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P, _P, _P, _P]

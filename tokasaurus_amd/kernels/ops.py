@@ -546,6 +546,44 @@ def sample(
     return ids, logprobs
 
 
+TOPK_MAX = 32  # places the top-k kernel ranks (TOPK_MAX of sample.hip)
+
+
+def topk_logprobs(logits: torch.Tensor, temperature: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """The ``k`` most probable tokens of every row (int32 [rows, k]) and their
+    log-probabilities under softmax(logits / T) (float32 [rows, k]; T 0 counts as 1),
+    most probable first, the lower index first among equal logits."""
+    _gpu(logits, temperature)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
+          "topk_logprobs: logits must be float32 [rows, vocab]")
+    rows, vocab = logits.shape
+    _need(temperature.dtype == torch.float32 and temperature.numel() == rows and temperature.is_contiguous(),
+          "topk_logprobs: temperature must be float32 [rows]")
+    _need(1 <= k <= min(TOPK_MAX, vocab), f"topk_logprobs: k={k} is not between 1 and {min(TOPK_MAX, vocab)}")
+    ids = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
+    logprobs = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
+    chunks = load("core").tk_sample_chunks(vocab)
+    n = max(rows, 1) * chunks
+    part = torch.empty((2 * n * k + 2 * n,), dtype=torch.float32, device=logits.device)
+    call(
+        "tk_topk_logprobs",
+        logits.data_ptr(),
+        logits.stride(0) if rows > 0 else vocab,
+        rows,
+        vocab,
+        temperature.data_ptr(),
+        k,
+        ids.data_ptr(),
+        logprobs.data_ptr(),
+        part[: n * k].data_ptr(),
+        part[n * k : 2 * n * k].data_ptr(),
+        part[2 * n * k : 2 * n * k + n].data_ptr(),
+        part[2 * n * k + n :].data_ptr(),
+        _stream(),
+    )
+    return ids, logprobs
+
+
 # --------------------------------------------------------------------------
 # bfloat16 matrix products on the matrix cores
 # --------------------------------------------------------------------------

@@ -5,7 +5,9 @@ The reference samples with a temperature only: ``top_p`` must be 1.0
 logit bias and best_of are rejected (tokasaurus/server/utils.py:459-531).
 Temperature 0 is greedy (tokasaurus/model/types.py:302-312).  The reference
 ignores a request's seed (tokasaurus/server/types.py:36); here it selects the
-request's stream of uniform numbers.
+request's stream of uniform numbers.  ``topk_logprobs`` asks for the most probable
+tokens of every step and their log-probabilities (tokasaurus/server/types.py:151),
+at most as many as the engine's ``max_topk_logprobs``.
 """
 
 from __future__ import annotations
@@ -20,6 +22,7 @@ class SamplingParams:
     max_tokens: int = 16
     ignore_eos: bool = False
     seed: int | None = None
+    topk_logprobs: int | None = None
 
     def __post_init__(self) -> None:
         if self.temperature < 0:
@@ -28,3 +31,5 @@ class SamplingParams:
             raise ValueError("top_p other than 1.0 is not supported")
         if self.max_tokens < 1:
             raise ValueError("max_tokens must be at least 1")
+        if self.topk_logprobs is not None and self.topk_logprobs < 1:
+            raise ValueError("topk_logprobs must be at least 1")
