@@ -118,7 +118,7 @@ def test_finalize_derives_and_checks():
 def test_settings_of_the_reference_that_are_not_built_are_refused():
     from tokasaurus_amd.config.engine_config import EngineConfig, OptionError
 
-    for kw, msg in ((dict(greedy_prefill=False), "paced prefill"), (dict(max_topk_logprobs=33), "between 1 and 32"), (dict(max_topk_logprobs=0), "between 1 and 32"),
+    for kw, msg in ((dict(prefill_round_up_multiple=0), "at least 1"), (dict(max_topk_logprobs=33), "between 1 and 32"), (dict(max_topk_logprobs=0), "between 1 and 32"),
                     (dict(log_level="chatty"), "logging level"), (dict(scheduling_steps_ahead=-1), "negative")):
         with pytest.raises(OptionError, match=msg):
             EngineConfig(kv_cache_num_tokens=1024, **kw).finalize()

@@ -76,6 +76,23 @@ def test_temperature_generation_config_b_in_portions_of_16(folders):
     assert engine.stats.steps > 130 // 16
 
 
+def test_paced_prefill_gives_the_plain_tokens(folders):
+    """greedy_prefill=F with a cache so small that requests wait: prompts go in paced
+    portions beside the decoding of others, and every completion is the plain one."""
+    cfg, _ = TINY["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 140 + n) for n in (9, 30, 21, 14, 26)]
+    engine = engine_for(folders, "A", greedy_prefill=False, prefill_round_up_multiple=4, kv_cache_num_tokens=80)
+    greedy = engine_for(folders, "A", kv_cache_num_tokens=80)
+    params = SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True)
+    done = engine.generate(prompts, params)
+    for prompt, c in zip(prompts, done):
+        want, _ = plain_generate(folders["A"], prompt, 7)
+        assert c.tokens == want
+    greedy.generate(prompts, params)
+    assert engine.stats.steps > greedy.stats.steps  # prompts were held back
+    assert engine.runner.manager.num_free_pages() == [80 // PAGE_A]
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 def test_ranked_tokens_and_their_logprobs(folders, graphs):
     """max_topk_logprobs=4: a request that asks for 3 gets every token's 3 most probable

@@ -13,10 +13,11 @@ from tokasaurus_amd.sampling import SamplingParams
 
 
 def make(num_pages=64, page_size=4, max_tokens_per_forward=32, max_seqs=8, eos=(), optimistic=False,
-         chunk=None, slots=None):
+         chunk=None, slots=None, greedy=True, multiple=16):
     cache = CacheManager([CacheGroup(CacheNeed(2, 16, 0), (0,))], num_pages, page_size, slots or max_seqs)
     s = Scheduler(cache, max_tokens_per_forward, max_seqs, max_num_tokens_per_request=10_000,
-                  eos_token_ids=eos, optimistic=optimistic, max_prefill_chunk=chunk, sanity_checks=True)
+                  eos_token_ids=eos, optimistic=optimistic, max_prefill_chunk=chunk, sanity_checks=True,
+                  greedy_prefill=greedy, prefill_round_up_multiple=multiple)
     return s, cache
 
 
@@ -287,3 +288,68 @@ def test_ranked_tokens_are_kept_only_as_far_as_a_request_asked():
     by_id = {r.id: r for r in done}
     assert by_id["a"].topk_ids == [[0, 50], [10, 50]] and by_id["a"].topk_logprobs == [[-0.1, -1.0]] * 2
     assert by_id["b"].topk_ids == [] and by_id["b"].completion == [7, 7]
+
+
+def paced_case(**kw):
+    """a (prompt 8, 9 tokens: 4 pages) and b (prompt 40, 5 tokens: 11 pages) run; c (prompt 24,
+    5 tokens: 7 pages) waits, since 20 pages leave only 5."""
+    s, cache = make(num_pages=20, page_size=4, max_tokens_per_forward=64, **kw)
+    s.submit(req("a", 8, 9)); s.submit(req("b", 40, 5)); s.submit(req("c", 24, 5))
+    return s
+
+
+def test_paced_prefill_by_hand():
+    s = paced_case(greedy=False, multiple=4)
+    d0 = s.schedule(); s.advance(d0)
+    # nothing decodes yet: exactly the first prompt (tokasaurus/manager/scheduler.py:616-619)
+    assert [(r.id, n) for r, n in d0.prefill] == [("a", 8)] and list(s.queued) == ["c"]
+    d1 = s.schedule()
+    # a ends at step 7, b (40 tokens at the last step's 8 a step: prompt done at step 4) at step 8.
+    # At step 7 c's 7 pages do not fit beside a and b (15 of 20): pace 40 / 8 = 5 tokens a step;
+    # at step 8, with a gone, c fits and nobody is left waiting.  5 goes up to 8.
+    assert [r.id for r in d1.decode] == ["a"] and [(r.id, n) for r, n in d1.prefill] == [("b", 8)]
+    assert s._paced_prefill() == 5.0
+    # always up, also from a multiple (scheduler.py:629-632)
+    s.prefill_round_up_multiple = 5
+    assert s._prefill_budget(1) == 10
+    # the same moment, prompts taken greedily: all of b
+    g = paced_case(greedy=True)
+    d0 = g.schedule(); g.advance(d0)
+    assert [(r.id, n) for r, n in d0.prefill] == [("a", 8), ("b", 40)]
+
+
+def test_paced_prefill_with_nobody_waiting_fills_the_budget():
+    s, _ = make(num_pages=64, max_tokens_per_forward=16, greedy=False)
+    s.submit(req("a", 4, 6)); s.submit(req("b", 30, 3))
+    d0 = s.schedule(); s.advance(d0)
+    assert [(r.id, n) for r, n in d0.prefill] == [("a", 4), ("b", 12)]  # the queue is empty: as fast as possible
+    d1 = s.schedule()
+    assert [(r.id, n) for r, n in d1.prefill] == [("b", 15)] and len(d1.decode) == 1
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_paced_prefill_changes_the_steps_and_no_completion(seed):
+    def workload(greedy):
+        rng = random.Random(seed)
+        P = rng.choice([2, 4, 16])
+        s, cache = make(num_pages=rng.choice([24, 40]), page_size=P, max_tokens_per_forward=rng.choice([16, 24]),
+                        max_seqs=rng.choice([3, 4, 8]), eos=(3,), greedy=greedy, multiple=rng.choice([1, 4, 16]))
+        total = cache.num_free_pages()[0]
+        for i in range(14):
+            plen, mt = rng.randint(1, 20), rng.randint(1, 12)
+            if math.ceil((plen + mt - 1) / P) <= total:
+                s.submit(req(f"r{i}", plen, mt, ignore_eos=(i % 5 == 0)))
+        return s, cache
+
+    def token_of(r, index):
+        return random.Random(f"{seed}/{r.id}/{index}").choice([3, 5, 6, 7, 8, 9])
+
+    results = []
+    for greedy in (True, False):
+        for ahead in (False, True):
+            s, cache = workload(greedy)
+            total = cache.num_free_pages()
+            results.append(drive(s, token_of, ahead))
+            assert cache.num_free_pages() == total and cache.slots.num_free == cache.slots.num_slots
+            assert s.num_bumps == 0
+    assert all(r == results[0] for r in results) and len(results[0]) > 0

@@ -38,8 +38,8 @@ class EngineConfig:
     max_tokens_per_forward: int = 8192
     max_seqs_per_forward: int = 1024
     max_num_tokens_per_request: int | None = None
-    prefill_round_up_multiple: int = 16  # rounds the paced prefill of the reference; without effect on the greedy one
-    greedy_prefill: bool = True  # the reference's default is F (paced prefill), which is not built here
+    prefill_round_up_multiple: int = 16  # rounds the paced prefill (greedy_prefill=F) up; without effect on the greedy one
+    greedy_prefill: bool = True  # F: prompts are paced so that new requests arrive as running ones end
 
     # --- outputs (tokasaurus/common_types.py:64-65)
     enable_chosen_logprobs: bool = True
@@ -87,8 +87,8 @@ class EngineConfig:
             raise OptionError("scheduling_steps_ahead must not be negative")
         # options of the reference whose other settings this engine does not build: say so
         # instead of going on as if they had been honoured
-        if not self.greedy_prefill:
-            raise OptionError("greedy_prefill=F (the reference's paced prefill) is not built: prompts take what the token budget leaves")
+        if self.prefill_round_up_multiple < 1:
+            raise OptionError("prefill_round_up_multiple must be at least 1")
         if self.max_topk_logprobs is not None and not 1 <= self.max_topk_logprobs <= MAX_TOPK_LOGPROBS:
             raise OptionError(f"max_topk_logprobs must be between 1 and {MAX_TOPK_LOGPROBS} (what the ranking kernel takes)")
         if self.log_level.upper() not in ("DEBUG", "INFO", "WARNING", "ERROR", "CRITICAL"):

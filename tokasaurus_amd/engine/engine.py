@@ -109,6 +109,8 @@ class Engine:
             optimistic=config.bump_city_population_me,
             max_prefill_chunk=config.max_prefill_chunk,
             sanity_checks=config.allocator_sanity_checks,
+            greedy_prefill=config.greedy_prefill,
+            prefill_round_up_multiple=config.prefill_round_up_multiple,
         )
         self.stats = Stats()
         self._next_id = 0

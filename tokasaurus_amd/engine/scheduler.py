@@ -89,8 +89,13 @@ class Scheduler:
         optimistic: bool = False,
         max_prefill_chunk: int | None = None,
         sanity_checks: bool = False,
+        greedy_prefill: bool = True,
+        prefill_round_up_multiple: int = 16,
     ):
         self.cache = cache
+        self.greedy_prefill = greedy_prefill
+        self.prefill_round_up_multiple = max(1, int(prefill_round_up_multiple))
+        self.last_num_prefill = 1 << 30  # prompt tokens of the last step that had any (manager/types.py:312)
         self.max_tokens_per_forward = max_tokens_per_forward
         self.max_seqs_per_forward = max_seqs_per_forward
         self.max_num_tokens_per_request = max_num_tokens_per_request
@@ -155,7 +160,7 @@ class Scheduler:
         self._make_room_for_decoding()
         self._admit()
         decode = list(self.decoding.values())
-        budget = self.max_tokens_per_forward - len(decode)
+        budget = self._prefill_budget(len(decode))
         prefill: list[tuple[Request, int]] = []
         for req in self.prefilling.values():
             if budget <= 0:
@@ -165,9 +170,73 @@ class Scheduler:
                 n = min(n, self.max_prefill_chunk)
             prefill.append((req, n))
             budget -= n
+        if prefill:
+            self.last_num_prefill = sum(n for _, n in prefill)  # manager.py:872-876
         if self.sanity_checks:
             self.cache.check()
         return Decision(prefill, decode)
+
+    def _prefill_budget(self, num_decoding: int) -> int:
+        """Prompt tokens for this step (tokasaurus/manager/scheduler.py:598-637): what the
+        token budget leaves when prompts are taken greedily or nobody waits in the queue;
+        the whole first prompt when nothing decodes; otherwise the paced amount, rounded up
+        to the next multiple of ``prefill_round_up_multiple``."""
+        most = self.max_tokens_per_forward - num_decoding
+        if not self.prefilling:
+            return 0
+        if self.greedy_prefill or not self.queued:
+            return most
+        if num_decoding == 0:
+            first = next(iter(self.prefilling.values()))
+            return min(most, len(first.prompt) - first.prompt_done)
+        pace = self._paced_prefill()
+        if pace == float("inf"):
+            return most
+        m = self.prefill_round_up_multiple
+        return min(most, int(pace + (m - pace % m)))  # scheduler.py:629-632: always up, also from a multiple
+
+    def _paced_prefill(self) -> float:
+        """Prompt tokens a step so that new work arrives as running requests end
+        (tokasaurus/manager/scheduler.py:433-538).  For every future step at which a running
+        request ends by length: the queued requests that can be admitted by then, first in
+        first out, beside the requests still running then; the prompt tokens outstanding by
+        then, over the steps until then; the slowest of these rates.  Infinite once the whole
+        queue fits.  A request counts with the pages of its whole life, as in admission here
+        (the reference counts the pages it expects, manager/types.py:94-104)."""
+        pages = {r.id: self.cache.blocks_for(r.max_cache_tokens()) for r in self.running()}
+        ends: list[tuple[int, Request]] = [(r.params.max_tokens - r.sampled - 1, r) for r in self.decoding.values()]
+        outstanding = 0
+        for r in self.prefilling.values():
+            outstanding += len(r.prompt) - r.prompt_done
+            prompt_ends = -(-outstanding // self.last_num_prefill) - 1  # scheduler.py:73-86
+            ends.append((prompt_ends + r.params.max_tokens - 1, r))
+        ends.sort(key=lambda e: e[0])
+        total = min(pool.num_pages for pool in self.cache.pools)
+        held = sum(pages.values())
+        queued = list(self.queued.values())
+        at, running = 0, len(ends)
+        added_pages = added_tokens = 0
+        slowest = float("inf")
+        i = 0
+        while i < len(ends):
+            step = ends[i][0]
+            # right before the requests that end at this step give their pages back
+            while at < len(queued) and running < self.max_seqs_per_forward:
+                need = self.cache.blocks_for(queued[at].max_cache_tokens())
+                if need > total - held - added_pages:
+                    break  # first in first out: nobody overtakes the head
+                added_tokens += len(queued[at].prompt)
+                added_pages += need
+                running += 1
+                at += 1
+            if at == len(queued):
+                break  # from here on everything fits: no later step slows the pace
+            slowest = min(slowest, (outstanding + added_tokens) / (step + 1))
+            running -= 1  # scheduler.py:536
+            while i < len(ends) and ends[i][0] == step:
+                held -= pages[ends[i][1].id]
+                i += 1
+        return slowest
 
     def _make_room_for_decoding(self) -> None:
         """Every decoding request needs room for one more token; when pages run
