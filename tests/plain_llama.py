@@ -128,7 +128,10 @@ def causal_attention(
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """nn.Linear without bias (llama.py:130-149): weight is [out, in]."""
+    """nn.Linear without bias (llama.py:130-149): weight is [out, in].  In bfloat16 the
+    product is summed in 32-bit and rounded once, as the reference's library does."""
+    if x.dtype == torch.bfloat16:
+        return (x.float() @ weight.float().T).to(torch.bfloat16)
     return x @ weight.T
 
 
@@ -192,15 +195,18 @@ def lm_head(x: torch.Tensor, w: dict[str, torch.Tensor], cfg: dict) -> torch.Ten
 # --------------------------------------------------------------------------
 
 
-def load_folder(folder: str | Path) -> tuple[dict, dict[str, torch.Tensor]]:
-    """config.json as a dict and every tensor of model.safetensors in 32-bit (tables of integers as they are)."""
+def load_folder(folder: str | Path, dtype: torch.dtype = torch.float32) -> tuple[dict, dict[str, torch.Tensor]]:
+    """config.json as a dict and every tensor of model.safetensors in 32-bit (tables of
+    integers as they are).  With ``dtype=torch.bfloat16`` the whole plain model computes as
+    the reference does in bfloat16 (every part keeps its input's dtype and does in 32-bit
+    what the reference does in 32-bit): the measure of what bfloat16 rounding alone costs."""
     folder = Path(folder)
     cfg = json.loads((folder / "config.json").read_text())
     weights = {}
     with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
         for name in f.keys():
             t = f.get_tensor(name)
-            weights[name] = t.to(torch.float32) if t.is_floating_point() else t
+            weights[name] = t.to(dtype) if t.is_floating_point() else t
     return cfg, weights
 
 

@@ -4,6 +4,7 @@ same requests can be compared with the plain implementation row by row."""
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 import plain_llama
@@ -59,6 +60,34 @@ def portions(rid: str, tokens: list[int], sizes: list[int]) -> list[dict]:
         at += n
         k += 1
     steps[-1]["end"] = [rid]
+    return steps
+
+
+def mixed_trace(reqs: dict[str, list[int]], seed: int, max_live: int = 4):
+    """Up to four live requests; portions of some beside single tokens of others; a
+    request may sit out a step; finished requests' pages go to later ones."""
+    rng = np.random.default_rng(seed)
+    waiting = list(reqs)
+    live: dict[str, int] = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
+            live[waiting.pop(0)] = 0
+        entries, ended = [], []
+        for rid in list(live):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue  # left out of this step
+            at, toks = live[rid], reqs[rid]
+            left = len(toks) - at
+            n = 1 if (left <= 12 or rng.random() < 0.4) else int(rng.choice([2, 3, 5, 8, 13, 21]))
+            n = min(n, left)
+            entries.append((rid, toks[at:at + n], list(range(n))))
+            live[rid] = at + n
+            if live[rid] == len(toks):
+                ended.append(rid)
+                del live[rid]
+        if entries:
+            steps.append({"entries": entries, "end": ended})
     return steps
 
 

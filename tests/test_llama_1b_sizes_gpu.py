@@ -1,0 +1,108 @@
+"""The layer sizes of Llama-3.2-1B (hidden 2048, 32 heads over 8 kv heads of 64, intermediate
+8192, a vocabulary of 128256, llama3 rotary scaling, tied head) with two layers and random
+weights: the sizes the kernels are tuned for, against the plain implementation, in 32-bit and
+in bfloat16, a long request with its last tokens one by one and mixed batches on few pages."""
+
+import pytest
+import torch
+
+import plain_llama
+from gpu_common import TOL
+from replay_helpers import compare, mixed_trace, run_steps
+from tiny_models import make_folder, random_tokens
+from tokasaurus_amd.engine.runner import ModelRunner
+
+pytestmark = pytest.mark.gpu
+
+CONFIG_1B_SIZES = {
+    "architectures": ["LlamaForCausalLM"],
+    "model_type": "llama",
+    "num_hidden_layers": 2,
+    "hidden_size": 2048,
+    "num_attention_heads": 32,
+    "num_key_value_heads": 8,
+    "intermediate_size": 8192,
+    "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {
+        "rope_type": "llama3",
+        "factor": 32.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 8192,
+    },
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 131072,
+}
+PAGE = 16
+LONG = 600
+MIXED = [90, 47, 130, 33, 71]
+# logits are compared at these places of the long request's first step, and at every later place
+LONG_WANT = [0, 1, 15, 16, 100, 255, 256, 511, 567]
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("llama_1b_sizes"), CONFIG_1B_SIZES, seed=3)
+    V = CONFIG_1B_SIZES["vocab_size"]
+    requests = {"long": random_tokens(LONG, V, 900)}
+    requests.update({f"m{i}": random_tokens(n, V, 910 + i) for i, n in enumerate(MIXED)})
+    cfg, w = plain_llama.load_folder(folder)
+    plain = {rid: plain_llama.forward_logits(cfg, w, toks) for rid, toks in requests.items()}
+    del w
+    # the plain model computing in bfloat16 as the reference does: what the rounding alone costs
+    cfg, w16 = plain_llama.load_folder(folder, torch.bfloat16)
+    plain16 = {rid: plain_llama.forward_logits(cfg, w16, toks) for rid, toks in requests.items()}
+    return folder, requests, plain, plain16
+
+
+def errors(got, plain, other=None):
+    """Root mean square and largest difference from the plain 32-bit logits over the rows of
+    ``got``, of ``got`` itself or of the same rows of ``other``."""
+    sq, n, worst = 0.0, 0, 0.0
+    for (rid, pos), row in got.items():
+        d = ((other[rid][pos] if other is not None else row) - plain[rid][pos]).double()
+        sq += float((d * d).sum())
+        n += d.numel()
+        worst = max(worst, float(d.abs().max()))
+    return (sq / n) ** 0.5, worst
+
+
+def long_steps(tokens):
+    head = LONG - 32
+    steps = [{"entries": [("long", tokens[:head], LONG_WANT)]}]
+    steps += [{"entries": [("long", [t], [0])]} for t in tokens[head:]]
+    steps[-1]["end"] = ["long"]
+    return steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_request_and_mixed_batches(model, dtype):
+    folder, requests, plain, plain16 = model
+    # room for the long request, or for the four longest of the mixed ones: pages are used again
+    runner = ModelRunner.from_folder(folder, dtype, page_size=PAGE, num_pages=-(-LONG // 64) * 64 // PAGE, max_slots=4)
+    got = run_steps(runner, long_steps(requests["long"]))
+    assert len(got) == len(LONG_WANT) + 32
+    mixed = {rid: toks for rid, toks in requests.items() if rid != "long"}
+    steps = mixed_trace(mixed, seed=5)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    got.update(run_steps(runner, steps))
+    assert len(got) == len(LONG_WANT) + 32 + sum(MIXED)
+    rms, worst = errors(got, plain)
+    print(f"{dtype}: rms error {rms:.3e}, largest {worst:.3e} against the plain 32-bit logits")
+    if dtype == "float32":
+        compare(got, plain, **TOL[dtype])
+    else:
+        # Six million logits through 2048-wide sums: the largest of so many rounding errors
+        # lies beyond what the tiny models' bound allows for a few thousand.  The measure here is
+        # the plain model computing in bfloat16 like the reference: the engine, which rounds in
+        # fewer places, must not be further from the 32-bit logits than that, row for row.
+        rms16, worst16 = errors(got, plain, plain16)
+        print(f"plain bfloat16: rms error {rms16:.3e}, largest {worst16:.3e}")
+        assert rms <= rms16 and worst <= worst16
+        for key, row in got.items():
+            r, _ = errors({key: row}, plain)
+            r16, _ = errors({key: row}, plain, plain16)
+            assert r <= 1.25 * r16, (key, r, r16)
+    assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]

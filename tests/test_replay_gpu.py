@@ -12,7 +12,7 @@ import torch
 
 import plain_llama
 from gpu_common import TOL
-from replay_helpers import compare, plain_rows, portions, run_steps, tail_one_by_one, whole
+from replay_helpers import compare, mixed_trace, plain_rows, portions, run_steps, tail_one_by_one, whole
 from tiny_models import TINY, random_tokens
 from tokasaurus_amd.cache import NoSpaceException
 from tokasaurus_amd.engine.batch import StepEntry
@@ -70,34 +70,6 @@ def test_portions_of_changing_size(folders, name, dtype):
         sizes = [[16, 7, 2, 5, 3], [2, 2, 31, 1, 4, 9], [3, 64, 2]][k % 3]
         got = run_steps(runner, portions(rid, toks, sizes))
         compare(got, ref, **TOL[dtype])
-
-
-def mixed_trace(reqs: dict[str, list[int]], seed: int, max_live: int = 4):
-    """Up to four live requests; portions of some beside single tokens of others; a
-    request may sit out a step; finished requests' pages go to later ones."""
-    rng = np.random.default_rng(seed)
-    waiting = list(reqs)
-    live: dict[str, int] = {}
-    steps = []
-    while waiting or live:
-        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
-            live[waiting.pop(0)] = 0
-        entries, ended = [], []
-        for rid in list(live):
-            if len(live) > 1 and rng.random() < 0.2:
-                continue  # left out of this step
-            at, toks = live[rid], reqs[rid]
-            left = len(toks) - at
-            n = 1 if (left <= 12 or rng.random() < 0.4) else int(rng.choice([2, 3, 5, 8, 13, 21]))
-            n = min(n, left)
-            entries.append((rid, toks[at:at + n], list(range(n))))
-            live[rid] = at + n
-            if live[rid] == len(toks):
-                ended.append(rid)
-                del live[rid]
-        if entries:
-            steps.append({"entries": entries, "end": ended})
-    return steps
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
