@@ -60,7 +60,17 @@ def parse() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--prefill-only", action="store_true", help="time only the prefill (for profiles); prints its record alone")
     p.add_argument("--eager", action="store_true", help="no HIP graphs")
+    p.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes (the default is the headline's)")
     return p.parse_args()
+
+
+# the other Llama shapes the reference is quoted on: for looking at the kernels at further sizes
+LLAMA_3B = dict(LLAMA_1B, num_hidden_layers=28, hidden_size=3072, num_attention_heads=24, num_key_value_heads=8,
+                intermediate_size=8192)
+LLAMA_8B = dict(LLAMA_1B, num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                intermediate_size=14336, tie_word_embeddings=False,
+                rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=8.0))
+SHAPES = {"1b": ("llama-3.2-1b-shape", LLAMA_1B), "3b": ("llama-3.2-3b-shape", LLAMA_3B), "8b": ("llama-3.1-8b-shape", LLAMA_8B)}
 
 
 def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int, context: int, use_graphs: bool):
@@ -183,7 +193,8 @@ def main() -> int:
         return 2
     import torch
 
-    cfgd = dict(LLAMA_1B)
+    model_name, shape = SHAPES[args.shape]
+    cfgd = dict(shape)
     model_layers = cfgd["num_hidden_layers"]
     if args.layers is not None:
         cfgd["num_hidden_layers"] = args.layers
@@ -206,7 +217,9 @@ def main() -> int:
     nbytes = decode_bytes(runner.model, cfgd, args.batch, mean_ctx, elem)
     achieved = nbytes / dt / 1e9
     out = {
-        "metric": "decode tok/s at batch 8 (Llama-3.2-1B shape, context 8192)",
+        "metric": f"decode tok/s at batch {args.batch} ({model_name}, context {args.context})"
+        if (args.shape, args.batch, args.context) != ("1b", 8, CONTEXT)
+        else "decode tok/s at batch 8 (Llama-3.2-1B shape, context 8192)",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -219,7 +232,7 @@ def main() -> int:
         "dtype": key,
         "data": "synthetic (seeded random weights and token ids)",
         "config": {
-            "model": "llama-3.2-1b-shape",
+            "model": model_name,
             "global_batch": args.batch,
             "seq_len": args.context,
             "parallelism": "single-gpu",
@@ -234,7 +247,7 @@ def main() -> int:
             "page_size": PAGE_SIZE,
             "tie_word_embeddings": cfgd["tie_word_embeddings"],
             "rope_theta": cfgd["rope_theta"],
-            "rope_scaling": "llama3 factor 32 low 1 high 4 orig 8192",
+            "rope_scaling": "llama3 factor {factor:g} low {low_freq_factor:g} high {high_freq_factor:g} orig {original_max_position_embeddings}".format(**cfgd["rope_scaling"]),
             "rms_norm_eps": cfgd["rms_norm_eps"],
             "hip_graphs": not args.eager,
         },
