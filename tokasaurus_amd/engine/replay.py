@@ -62,7 +62,9 @@ def run(args: argparse.Namespace, lines=None, out=None) -> int:
                 arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                 np.ascontiguousarray(arr).tofile(out_dir / f"{rec['step']}.f32")
         for rid in rec.get("end", []):
-            runner.release(str(rid))
+            # a request that never held anything (or was ended before) has nothing to give back
+            if str(rid) in runner.manager.requests:
+                runner.release(str(rid))
         print(f"done {rec['step']}", file=out, flush=True)
     return 0
 
