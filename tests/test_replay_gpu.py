@@ -194,3 +194,31 @@ def test_trace_run_program(folders, tmp_path, dtype):
         assert arr.shape[0] == len(rows)
         got = {key: torch.from_numpy(arr[i].copy()) for i, key in enumerate(rows)}
         compare(got, ref, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_context_of_twenty_thousand_tokens(tmp_path, dtype):
+    """One layer of configuration C over 20,000 tokens in portions of up to 8,192, then eight
+    tokens one by one: more than a thousand pages in one block table, keys split many
+    ways.  Logits are compared at every 997th place, at the first places and at the last 48."""
+    from tiny_models import CONFIG_C, make_folder
+
+    N = 20000
+    cfg = dict(CONFIG_C, num_hidden_layers=1, max_position_embeddings=32768)
+    folder = make_folder(tmp_path / "long", cfg, seed=4)
+    toks = random_tokens(N + 8, cfg["vocab_size"], 1)
+    pcfg, w = plain_llama.load_folder(folder)
+    ref = {"x": plain_llama.forward_logits(pcfg, w, toks)}
+    runner = ModelRunner.from_folder(folder, dtype, page_size=16, num_pages=-(-(N + 8) // 64) * 64 // 16, max_slots=4)
+    steps, at = [], 0
+    for size in [8192, 5000, 3, 8192]:
+        n = min(size, N - at)
+        want = [i for i in range(n) if (at + i) % 997 == 0 or at + i < 3 or at + i >= N - 40]
+        steps.append({"entries": [("x", toks[at:at + n], want)]})
+        at += n
+    assert at == N
+    steps += [{"entries": [("x", [t], [0])]} for t in toks[N:]]
+    steps[-1]["end"] = ["x"]
+    got = run_steps(runner, steps)
+    assert len(got) > 60
+    compare(got, ref, **TOL[dtype])
