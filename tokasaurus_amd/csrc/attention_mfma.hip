@@ -208,7 +208,12 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int NW = blockDim.x >> 6;
   const int r = lane & 15, q = lane >> 4;
-  const int tile = blockIdx.x, kvh = blockIdx.y;
+  // Workgroups go to the chip's eight dies in turn, each with a cache of its own.  Prompts
+  // (two row tiles): kv head fastest, so a die serves few kv heads and keeps their keys and
+  // values, which every tile of the request reads again, to itself.  Decoded tokens read
+  // their keys once: tile fastest, as measured.
+  const int kvh = RT == 2 ? blockIdx.x % a.nkv : blockIdx.x / a.n_tiles;
+  const int tile = RT == 2 ? blockIdx.x / a.nkv : blockIdx.x % a.n_tiles;
   const TileRange t = tile_range(a, tile, RT);
   const int s = t.s_first + blockIdx.z;
   if (s > t.s_last) return;
@@ -515,7 +520,7 @@ static bool launch_attn(const AttnArgs& a, int grid_splits, int nw, hipStream_t 
   if (lds > 64 * 1024 &&
       hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return false;
-  hipLaunchKernelGGL(kernel, dim3(a.n_tiles, a.nkv, grid_splits), dim3(64 * nw), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(a.n_tiles * a.nkv, 1, grid_splits), dim3(64 * nw), lds, stream, a);
   return true;
 }
 
