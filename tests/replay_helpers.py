@@ -107,3 +107,25 @@ def compare(got, want_rows: dict[str, torch.Tensor], atol: float, rtol: float) -
             )
         worst = max(worst, float(err.max()))
     return worst
+
+
+def compare_with_bfloat16_measure(got, plain: dict[str, torch.Tensor], plain16: dict[str, torch.Tensor],
+                                  atol: float, rtol: float) -> float:
+    """For models wider than the tiny ones, whose rounding errors outgrow a fixed bound: a
+    row of bfloat16 logits passes when it is within the bound, or else when it is less than
+    twice as far from the plain 32-bit row (root mean square) as the plain model computing
+    in bfloat16 is.  A wrong key or page moves a row many times further than rounding does.
+    Returns the largest ratio seen among the rows beyond the bound (0 if none)."""
+    worst = 0.0
+    for (rid, pos), row in sorted(got.items()):
+        ref = plain[rid][pos]
+        err = (row - ref).double()
+        if bool((err.abs() <= atol + rtol * ref.abs()).all()):
+            continue
+        err16 = (plain16[rid][pos] - ref).double()
+        ratio = float(err.pow(2).mean().sqrt() / err16.pow(2).mean().sqrt().clamp_min(1e-12))
+        if ratio >= 2.0:
+            raise AssertionError(f"request {rid} position {pos}: {ratio:.2f} times as far from the plain logits as "
+                                 f"the plain model in bfloat16 (largest error {float(err.abs().max()):.3e})")
+        worst = max(worst, ratio)
+    return worst
