@@ -4,7 +4,9 @@ from __future__ import annotations
 
 import pytest
 
+import plain_llama
 from tiny_models import TINY, make_folder
+from tokasaurus_amd.sampling import uniform_for
 
 # Logits of the tiny models are of order 1.  In 32-bit the engine and the plain
 # implementation differ by the order of summation only.  In bfloat16 every
@@ -20,3 +22,19 @@ TOL = {
 def folders(tmp_path_factory):
     root = tmp_path_factory.mktemp("models")
     return {name: make_folder(root / name, cfg, seed=11 + i) for i, (name, (cfg, _)) in enumerate(sorted(TINY.items()))}
+
+
+def plain_generate(folder, prompt, max_tokens, temperature=0.0, engine_seed=0, request_seed=0, eos=()):
+    """Token by token with the whole sequence recomputed; the same uniform numbers as the engine draws."""
+    cfg, w = plain_llama.load_folder(folder)
+    ids, out, lps = list(prompt), [], []
+    for i in range(max_tokens):
+        logits = plain_llama.forward_logits(cfg, w, ids)[-1]
+        u = uniform_for(engine_seed, request_seed, i) if temperature > 0 else 0.0
+        tok, lp = plain_llama.sample(logits, temperature, u)
+        out.append(tok)
+        lps.append(lp)
+        ids.append(tok)
+        if tok in eos:
+            break
+    return out, lps

@@ -11,6 +11,7 @@ import pytest
 import torch
 
 import plain_llama
+from gpu_common import plain_generate
 from tiny_models import CONFIG_A, PAGE_A, PAGE_B, TINY, make_folder, random_tokens
 from tokasaurus_amd import EngineConfig, SamplingParams
 from tokasaurus_amd.engine.engine import Engine
@@ -19,22 +20,6 @@ from tokasaurus_amd.sampling import uniform_for
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-
-
-def plain_generate(folder, prompt, max_tokens, temperature=0.0, engine_seed=0, request_seed=0, eos=()):
-    """Token by token with the whole sequence recomputed; the same uniform numbers as the engine draws."""
-    cfg, w = plain_llama.load_folder(folder)
-    ids, out, lps = list(prompt), [], []
-    for i in range(max_tokens):
-        logits = plain_llama.forward_logits(cfg, w, ids)[-1]
-        u = uniform_for(engine_seed, request_seed, i) if temperature > 0 else 0.0
-        tok, lp = plain_llama.sample(logits, temperature, u)
-        out.append(tok)
-        lps.append(lp)
-        ids.append(tok)
-        if tok in eos:
-            break
-    return out, lps
 
 
 def engine_for(folders, name, dtype="float32", **kw):

@@ -9,9 +9,11 @@ import pytest
 import torch
 
 import plain_llama
-from gpu_common import TOL
+from gpu_common import TOL, plain_generate
 from replay_helpers import compare, compare_with_bfloat16_measure, mixed_trace, plain_rows, run_steps
 from tiny_models import make_folder, random_tokens
+from tokasaurus_amd import EngineConfig, SamplingParams
+from tokasaurus_amd.engine.engine import Engine
 from tokasaurus_amd.engine.runner import ModelRunner
 
 pytestmark = pytest.mark.gpu
@@ -70,3 +72,39 @@ def test_a_random_configuration_in_mixed_batches(tmp_path, seed):
         else:
             compare_with_bfloat16_measure(got, plain, plain16, **TOL[dtype])
         assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
+
+
+@pytest.mark.parametrize("seed", [2, 8, 13, 21, 22, 23])
+def test_generation_under_random_options(tmp_path, seed):
+    """A random configuration under random engine options (page and cache size, budgets,
+    portions, optimistic admission, paced prompts, a step ahead or not, recorded steps or not)
+    and random sampling options, in 32-bit: every completion is the plain one's."""
+    rng = random.Random(seed)
+    cfg = random_config(rng)
+    cfg["num_hidden_layers"] = min(cfg["num_hidden_layers"], 2)
+    page = rng.choice([4, 8, 16, 32])
+    folder = make_folder(tmp_path / "m", cfg, seed=seed)
+    n = rng.randint(3, 9)
+    prompts = [random_tokens(rng.randint(1, 90), cfg["vocab_size"], 77 * seed + i) for i in range(n)]
+    params = [SamplingParams(temperature=rng.choice([0.0, 0.0, 0.7, 1.3]), max_tokens=rng.randint(1, 14), ignore_eos=True,
+                             seed=rng.randint(0, 999), topk_logprobs=rng.choice([None, 2])) for _ in range(n)]
+    need = max(len(p) + sp.max_tokens for p, sp in zip(prompts, params))
+    tokens = -(-rng.randint(need, 4 * need) // 64) * 64
+    options = dict(model=str(folder), dtype="float32", page_size=page, kv_cache_num_tokens=tokens,
+                   max_seqs_per_forward=rng.choice([2, 4, 8]), max_tokens_per_forward=rng.choice([16, 48, 128]),
+                   max_prefill_chunk=rng.choice([None, 3, 16]), bump_city_population_me=rng.random() < 0.4,
+                   greedy_prefill=rng.random() < 0.6, prefill_round_up_multiple=rng.choice([1, 4, 16]),
+                   scheduling_steps_ahead=rng.choice([0, 8]), use_hipgraphs=rng.random() < 0.7,
+                   allocator_sanity_checks=True, seed=seed, max_topk_logprobs=3)
+    print(f"seed {seed}: {cfg}\n{options}")
+    engine = Engine(EngineConfig(**options))
+    done = engine.generate(prompts, params)
+    for c, prompt, sp in zip(done, prompts, params):
+        want, want_lp = plain_generate(folder, prompt, sp.max_tokens, temperature=sp.temperature, engine_seed=seed,
+                                       request_seed=sp.seed)
+        assert c.tokens == want
+        assert torch.allclose(torch.tensor(c.logprobs), torch.tensor(want_lp), atol=2e-4)
+        assert (c.topk_ids is None) == (sp.topk_logprobs is None)
+        if c.topk_ids is not None:
+            assert [len(t) for t in c.topk_ids] == [2] * len(c.tokens)
+    assert engine.runner.manager.num_free_pages() == [p.num_pages for p in engine.runner.manager.pools]
