@@ -130,28 +130,50 @@ def test_bfloat16_generation_follows_the_plain_one(folders, name):
             ids.append(tok)
 
 
-@pytest.mark.parametrize("live, lengths", [(3, (30, 8, 55, 21, 40)), (40, tuple(5 + (7 * i) % 23 for i in range(44)))])
-def test_recorded_and_eager_decode_steps_agree(folders, live, lengths):
-    """The same requests with and without recorded steps, several replays with eager
-    work (prompt portions of later requests) between them: the same tokens.  With 40
-    live requests some steps have more rows than the weight-streaming product takes on:
-    those hold library products and are never recorded, the smaller ones are."""
-    cfg, _ = TINY["C"]
+def recorded_against_eager(folder, page, cfg, live, lengths, max_tokens, budget=None, padded=False):
+    """The same requests through an engine with recorded decode steps and one without; returns
+    the sizes that were recorded.  Requests end at different lengths, so the batch shrinks
+    through the recorded sizes, each replayed several times with eager steps (prompt portions
+    of later requests, and steps of sizes not yet recorded) between them; every replay's
+    tokens and log-probabilities are compared with the eager run's.  ``padded``: the eager
+    engine pads its decode steps as the recorded ones are padded and launches the same kernels
+    one by one (the library sums in another order for 48 rows than for 37, which at a flat
+    distribution over a large vocabulary moves a sampled token to its neighbour)."""
     prompts = [random_tokens(n, cfg["vocab_size"], 90 + n + i) for i, n in enumerate(lengths)]
-    results = []
+    params = [SamplingParams(temperature=0.7, max_tokens=max_tokens(i), ignore_eos=True, seed=3 + i) for i in range(len(lengths))]
+    results, sizes = [], set()
     for graphs in (True, False):
-        engine = engine_for(folders, "C", dtype="bfloat16", use_hipgraphs=graphs, max_seqs_per_forward=live,
-                            max_tokens_per_forward=max(32, live + 16), kv_cache_num_tokens=4096)
-        done = engine.generate(prompts, SamplingParams(temperature=0.7, max_tokens=20, ignore_eos=True, seed=3))
+        engine = Engine(EngineConfig(
+            model=str(folder), dtype="bfloat16", page_size=page, use_hipgraphs=graphs or padded, max_seqs_per_forward=live,
+            max_tokens_per_forward=budget or max(32, live + 16), kv_cache_num_tokens=16384, allocator_sanity_checks=True))
+        if padded and not graphs:
+            engine.runner.capture_graphs = False
+        done = engine.generate(prompts, params)
         results.append([(c.tokens, c.logprobs) for c in done])
-        assert bool(engine.runner.recorded) == graphs
         if graphs:
-            from tokasaurus_amd.kernels import ops
-
-            assert max(size for size, _ in engine.runner.recorded) == min(live, ops.SKINNY_ROWS)
+            sizes = {size for size, _ in engine.runner.recorded}
+            assert sizes and all(step.captured for step in engine.runner.recorded.values())
+        else:
+            assert not any(step.captured for step in engine.runner.recorded.values())
     for (ta, la), (tb, lb) in zip(*results):
         assert ta == tb
         assert torch.allclose(torch.tensor(la), torch.tensor(lb), atol=1e-5)
+    return sizes
+
+
+@pytest.mark.parametrize("live, count", [(3, 5), (40, 44), (128, 140)])
+def test_recorded_and_eager_decode_steps_agree(folders, live, count):
+    """With 40 and 128 live requests the recorded steps hold library products (more rows than
+    the weight-streaming product takes on); with 128 every recorded size from 48 to 128 rows
+    is replayed."""
+    cfg, page = TINY["C"]
+    lengths = [5 + (7 * i) % 23 for i in range(count)]
+    # with 128 live requests the prompts go in within three steps, so that all of them decode together
+    sizes = recorded_against_eager(folders["C"], page, cfg, live, lengths, lambda i: 6 + (5 * i) % 31,
+                                   budget=1024 if live == 128 else None)
+    assert max(sizes) >= min(live, count) - 15
+    if live == 128:
+        assert {48, 64, 80, 96, 112, 128} <= sizes
 
 
 def test_finishing_on_an_end_token_and_on_length(folders, tmp_path):

@@ -106,3 +106,15 @@ def test_long_request_and_mixed_batches(model, dtype):
             r16, _ = errors({key: row}, plain, plain16)
             assert r <= 1.25 * r16, (key, r, r16)
     assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
+
+
+def test_recorded_steps_with_library_products_agree_with_eager_ones(model):
+    """At these sizes the library picks other kernels than for the tiny models: every recorded
+    size up to 128 rows, replayed with eager steps between, against an eager run."""
+    from test_engine_gpu import recorded_against_eager
+
+    folder = model[0]
+    lengths = [3 + (5 * i) % 17 for i in range(136)]
+    sizes = recorded_against_eager(folder, PAGE, CONFIG_1B_SIZES, 128, lengths, lambda i: 6 + (3 * i) % 23, budget=1024,
+                                   padded=True)
+    assert {32, 48, 64, 80, 96, 112, 128} <= sizes

@@ -123,6 +123,7 @@ class RecordedDecodeStep:
         # cycle, or they would be freed by the cyclic collector at a time of its choosing,
         # possibly while another step is being recorded, when memory must not be released
         self.size = size
+        self.captured = runner.capture_graphs
         self.num_ranked = runner.topk_logprobs
         model, storage, manager = runner.model, runner.storage, runner.manager
         self.model, self.storage, self.manager = model, storage, manager
@@ -178,12 +179,13 @@ class RecordedDecodeStep:
                 self._forward()
             torch.cuda.current_stream().wait_stream(stream)
             torch.cuda.synchronize()
-            self.graph = torch.cuda.CUDAGraph()
-            # recorded steps run one at a time and their results are read before the next step:
-            # they share one pool of memory
-            with torch.cuda.graph(self.graph, pool=runner.graph_pool):
-                self.logits, self.ids, self.logprobs, self.topk = self._forward()
-            torch.cuda.synchronize()
+            if self.captured:
+                self.graph = torch.cuda.CUDAGraph()
+                # recorded steps run one at a time and their results are read before the next step:
+                # they share one pool of memory
+                with torch.cuda.graph(self.graph, pool=runner.graph_pool):
+                    self.logits, self.ids, self.logprobs, self.topk = self._forward()
+                torch.cuda.synchronize()
         finally:
             if was_enabled:
                 gc.enable()
@@ -241,7 +243,11 @@ class RecordedDecodeStep:
         self._fill(token_ids, positions, slots, out_slots, temps, us)
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
-        self.graph.replay()
+        if self.captured:
+            self.graph.replay()
+        else:
+            # the same padded step launched kernel by kernel: what a replay must reproduce bit for bit
+            self.logits, self.ids, self.logprobs, self.topk = self._forward()
         out = StepOutput(self.logits[:n], self.ids[:n], self.logprobs[:n] if self.logprobs is not None else None)
         if self.topk is not None:
             out.topk_ids, out.topk_logprobs = self.topk[0][:n], self.topk[1][:n]
@@ -279,12 +285,14 @@ class ModelRunner:
             self.groups, num_pages, page_size, max_slots, max_blocks_per_request=-(-limit // page_size)
         )
         self.use_graphs = use_graphs
-        # Only this engine's own kernels go into a recording.  In bfloat16, steps of more rows
-        # than the weight-streaming product takes on hold library products, which may keep
-        # work memory that they clear in ways a replay does not repeat: such steps run eagerly
-        # (the step launched ahead hides their launches; measured 1 to 2 % slower at 40 and 64 rows).
-        if model.dtype == torch.bfloat16:
-            graph_max_size = min(graph_max_size, ops.SKINNY_ROWS)
+        # False (set by tests before the first decode step): recorded steps keep their padded
+        # shapes and buffers but launch their kernels one by one instead of replaying a graph
+        self.capture_graphs = True
+        # Steps of more rows than the weight-streaming product takes on hold library products.
+        # They are recorded too: at short contexts an eager step of 40 to 128 rows is bound by the
+        # host's launches and takes up to twice as long (measured: 3.2 against 1.6 ms at 40 rows
+        # and 1,024 tokens of context).  The tests replay every recorded size several times with
+        # eager steps between and compare each replay's tokens with an eager run's.
         largest = min(graph_max_size, max(max_slots, 1))
         self.graph_sizes = [b for b in graph_buckets(graph_max_size, graph_step) if b <= largest] if use_graphs else []
         if use_graphs and largest not in self.graph_sizes:
