@@ -591,9 +591,10 @@ def topk_logprobs(logits: torch.Tensor, temperature: torch.Tensor, k: int) -> tu
 EPI_STORE, EPI_RESIDUAL, EPI_SWIGLU, EPI_F32, EPI_ROPE = 0, 1, 2, 3, 4
 SKINNY_MAX_ROWS = 128  # rows the weight-streaming kernel takes
 # Rows up to which it is the faster product.  Measured on an MI355X for the layer shapes of a
-# 1B model: at 32 rows it ties with the library product followed by the kernels it fuses away
-# (rotation and append, SwiGLU, norms); at 64 rows the library is a third faster.
-SKINNY_ROWS = 32
+# 1B model, whole recorded decode steps at a context of 1,024: at 8 and 16 rows 19 and 11 %
+# faster than the library product followed by the kernels it fuses away (rotation and append,
+# SwiGLU, norms); at 24 and 32 rows 12 % slower, at 64 rows a third.
+SKINNY_ROWS = 16
 
 
 class _GemmExtra(ctypes.Structure):
