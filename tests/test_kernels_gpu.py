@@ -441,7 +441,7 @@ def test_rope_table():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 8, 64, 16), (6, 2, 48, 16)])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 4), (3, 1, 32, 8), (8, 8, 64, 16), (6, 2, 48, 16), (5, 5, 40, 8), (2, 1, 128, 64)])
 def test_rope_append(dtype, shape):
     """Rotation of q and k against the plain formula, and the place of every key and value in the pages."""
     import plain_llama

@@ -310,9 +310,13 @@ TK_API int tk_rope_table(const float* inv_freq, float* cos_t, float* sin_t, int 
 // rope_append: for each token rotate its query heads in place, rotate its key
 // heads and store them, and store its value heads, in the token's page.
 //   qkv row: [nq*d | nkv*d | nkv*d]  (only the first part when !write_cache)
-//   K pages: [page][kv head][P][d]       V pages: [page][kv head][d][P]
+//   K pages: [page][kv head][d / 8][P][8]    V pages: [page][kv head][P / 4][d][4]
+//   (key_offset and value_offset of common.h)
 // Lane j pairs with lane j + d/2; the rotation is computed in 32-bit.
 // When cos_t is null the heads are stored unrotated (no position encoding).
+// One workgroup a token, an element (pair) a thread: a variant that moved 16 bytes a thread
+// was measured no faster (12.5 against 11.5 us for 2,048 tokens of the 1B shape): the
+// kernel waits for its chain of loads (position, table entry, row), not for its bytes.
 // --------------------------------------------------------------------------
 template <typename T>
 __global__ void rope_append_kernel(T* __restrict__ qkv, int row_stride,
