@@ -598,6 +598,9 @@ SKINNY_MAX_ROWS = 128  # rows the weight-streaming kernel takes
 # faster than the library product followed by the kernels it fuses away (rotation and append,
 # SwiGLU, norms); at 24 and 32 rows 12 % slower, at 64 rows a third.
 SKINNY_ROWS = 16
+# The stacked q, k, v product with rotation and append in its epilogue replaces two kernels of
+# the library path and has a short inner size: it stays ahead up to 32 rows (4 % of a step).
+SKINNY_ROPE_ROWS = 32
 
 
 class _GemmExtra(ctypes.Structure):

@@ -127,7 +127,8 @@ class Linear:
         append of k and v to the pages in its epilogue; returns q [M, nq*d], or None when
         that kernel does not take this case (the caller then does the steps one by one)."""
         m = (x.x if isinstance(x, Normed) else x).shape[0]
-        if not self._fast(m) or rope.head_dim % 2:
+        fits = self.weight.dtype == torch.bfloat16 and 0 < m <= ops.SKINNY_ROPE_ROWS and self._aligned()
+        if not fits or rope.head_dim % 2:
             return None
         prenorm, eps = None, 0.0
         if isinstance(x, Normed):
