@@ -135,9 +135,10 @@ def time_decode(runner, args, batch: int, ctx: int, steps: int, warmup: int) -> 
     engine = make_engine(runner, args, max_seqs=max(batch, 1))
     vocab = runner.model.spec.vocab_size
     # Prompts are prefilled by the engine under its token budget, so the first
-    # sequences already decode while the last are prefilled: `batch` + 8 tokens of
-    # slack keep every sequence within `ctx` when the timed steps end.
-    prompt_len = ctx - steps - warmup - batch - 8
+    # sequences already decode while the last are prefilled: as many tokens of slack as
+    # that takes steps (and 8 more) keep every sequence within `ctx` when the timed steps end.
+    prefill_steps = -(-batch * ctx // (8192 - batch)) + batch
+    prompt_len = ctx - steps - warmup - prefill_steps - 8
     g = torch.Generator().manual_seed(batch)
     for _ in range(batch):
         prompt = torch.randint(0, vocab, (prompt_len,), generator=g).tolist()
