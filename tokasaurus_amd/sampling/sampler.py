@@ -6,14 +6,11 @@ softmax(logits / T) by inverse CDF with one uniform number per row.  The
 reference takes that number from the global generator (llama.py:365); here it is
 a pure function of (engine seed, request seed, index of the token in the
 completion), so a request's tokens do not depend on what else was in the batch
-and a request that is restarted draws the same tokens again.
+and a request that is restarted draws the same tokens again.  The kernels are
+``ops.sample`` and ``ops.topk_logprobs``; the step function calls them with the step's rows.
 """
 
 from __future__ import annotations
-
-import torch
-
-from tokasaurus_amd.kernels import ops
 
 _MASK = (1 << 64) - 1
 
@@ -30,30 +27,3 @@ def uniform_for(engine_seed: int, request_seed: int, index: int) -> float:
     """A number in [0, 1) with 24 random bits, fixed by its three arguments."""
     h = _mix(_mix(_mix(engine_seed & _MASK) ^ (request_seed & _MASK)) ^ (index & _MASK))
     return (h >> 40) / float(1 << 24)
-
-
-class Sampler:
-    def __init__(self, device: torch.device, want_logprobs: bool = True):
-        self.device = device
-        self.want_logprobs = want_logprobs
-
-    def sample(
-        self,
-        logits: torch.Tensor,
-        temperatures: list[float],
-        uniforms: list[float],
-        slots: list[int] | None = None,
-        last_token: torch.Tensor | None = None,
-    ) -> tuple[torch.Tensor, torch.Tensor | None]:
-        """Token ids and log-probabilities (device tensors) for every row; when
-        ``slots`` is given each row's token is also written to its slot."""
-        rows = logits.shape[0]
-        assert len(temperatures) == rows and len(uniforms) == rows
-        params = torch.tensor([temperatures, uniforms], dtype=torch.float32).to(self.device)
-        slot_t = None
-        if slots is not None:
-            slot_t = torch.tensor(slots, dtype=torch.int32).to(self.device)
-        return ops.sample(
-            logits, params[0], params[1], slot_t, last_token if slots is not None else None,
-            want_logprobs=self.want_logprobs,
-        )
