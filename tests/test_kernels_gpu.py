@@ -86,6 +86,37 @@ def test_paged_attention(kind, case_id):
     assert not bad.any(), f"first wrong row {int(bad.any(1).nonzero()[0])}, largest error {float(err.max()):.3e}"
 
 
+@pytest.mark.parametrize("kind", ["generic_f32", "mfma", "mfma_pairs"])
+@pytest.mark.parametrize("window", [0, 600])
+def test_attention_finds_one_far_key(kind, window):
+    """One key among 1,500 answers the query (its score stands out by far), the others are
+    noise: the output is that key's value.  The key lies at the first and the last place, on
+    both sides of a page's edge and of a split's edge, and at the window's edge: just inside
+    it is found, just outside it is not."""
+    nq, nkv, d, page, kv_len = 4, 2, 64, 16, 1500
+    last = kv_len - 1
+    inside = [0, 15, 16, 511, 512, 1023, 1024, last - 1, last] if window == 0 else [last - window + 1, last - window + 2, 1023, 1024, last]
+    outside = [] if window == 0 else [last - window, last - window - 1, 0]
+    dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
+    for target in inside + outside:
+        case = make_paged_case([1], [kv_len], nq, nkv, d, page, seed=target, dtype=dtype, sharp=0.05)
+        k = case["k"][0]  # [kv_len, nkv, d]
+        q = case["q"].view(1, nq, d).clone()
+        for h in range(nq):
+            key = k[target, h // (nq // nkv)]
+            q[0, h] = key * (40.0 * d ** 0.5 / float(key.pow(2).sum()))  # a score of 40 against scores near 0
+        case["q"] = q.view(1, nq * d).to(dtype).float()
+        if kind == "generic_f32":
+            got = run_attention(kind, case, [1], [kv_len], nq, nkv, d, page, window)
+        else:
+            got = run_attention(kind, case, [1], [kv_len], nq, nkv, d, page, window, split=512 if kind == "mfma" else 4096,
+                                row_tiles=2 if kind == "mfma_pairs" else 1, pair=kind == "mfma_pairs")
+        got = got.float().cpu().view(nq, d)
+        want = torch.stack([case["v"][0][target, h // (nq // nkv)] for h in range(nq)])
+        close = torch.allclose(got, want, atol=3e-2, rtol=3e-2)
+        assert close == (target in inside), (target, float((got - want).abs().max()))
+
+
 def test_attention_splits_agree():
     """The same decode with different splits: equal beyond rounding of the merge."""
     q_lens, kv_lens, nq, nkv, d, page = [1, 1], [2000, 777], 8, 2, 64, 16
