@@ -522,7 +522,8 @@ def test_rope_append(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("mnk", [(1, 1000, 96), (37, 77, 130), (130, 64, 64), (5, 512, 2048)])
+@pytest.mark.parametrize("mnk", [(1, 1000, 96), (37, 77, 130), (130, 64, 64), (5, 512, 2048), (16, 77, 130), (9, 333, 240),
+                                 (32, 18, 4100), (33, 18, 260)])
 def test_gemm_generic(dtype, mnk):
     from tokasaurus_amd.kernels import ops
 

@@ -1,9 +1,93 @@
 // C[M,N] = A[M,K] * W[N,K]^T (+ residual[M,N]) with plain 32-bit multiply-adds:
 // the matrix product of the true 32-bit path, and the fallback of the bfloat16
 // path for shapes the MFMA kernels refuse.  Operands are row-major with K
-// contiguous; any M, N, K.  Each output element sums its K products in
-// ascending k, whatever M is, so a row's result does not depend on the batch.
+// contiguous; any M, N, K.  Two kernels: tiles of 64 x 64 through LDS, each output
+// summing its K products in ascending k; and, for up to GR_MAX_ROWS rows (decode), one
+// that streams the weights: a wavefront owns GR_COLS output columns, its lanes cut K
+// between them and add up at the end.  In both the order of an output's additions is
+// fixed by K alone, so a row's result does not depend on what else is in the batch
+// beyond which of the two kernels the batch's size selects (rounding).
 #include "common.h"
+
+#define GR_COLS 4
+#define GR_MAX_ROWS 32
+
+// Four consecutive elements as 32-bit floats: one 16-byte load where T is float and the
+// caller found sizes and addresses aligned, else element by element (k may run past K).
+template <typename T, bool VEC>
+__device__ __forceinline__ void load4(const T* row, int k, int K, float out[4]) {
+  if constexpr (VEC) {
+    const float4 v = *(const float4*)(row + k);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = (k + i < K) ? to_f32<T>(row[k + i]) : 0.f;
+  }
+}
+
+template <typename T, typename TO, int MB, bool VEC>
+__global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A, int lda,
+                                                        const T* __restrict__ W,
+                                                        TO* __restrict__ C, int ldc,
+                                                        const T* __restrict__ residual, int ldr,
+                                                        int M, int N, int K) {
+  const int lane = threadIdx.x & (TK_WAVE - 1), wave = threadIdx.x / TK_WAVE;
+  const int n0 = (blockIdx.x * (256 / TK_WAVE) + wave) * GR_COLS;
+  const int m0 = blockIdx.y * MB;
+  if (n0 >= N) return;
+  float acc[MB][GR_COLS];
+#pragma unroll
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int c = 0; c < GR_COLS; ++c) acc[m][c] = 0.f;
+  for (int k = lane * 4; k < K; k += TK_WAVE * 4) {
+    float w[GR_COLS][4];
+#pragma unroll
+    for (int c = 0; c < GR_COLS; ++c) load4<T, VEC>(W + (size_t)min(n0 + c, N - 1) * K, k, K, w[c]);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      if (m0 + m < M) {  // the same for every lane
+        float a[4];
+        load4<T, VEC>(A + (size_t)(m0 + m) * lda, k, K, a);
+#pragma unroll
+        for (int c = 0; c < GR_COLS; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[m][c] = fmaf(a[i], w[c][i], acc[m][c]);
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    if (m0 + m >= M) continue;
+#pragma unroll
+    for (int c = 0; c < GR_COLS; ++c) {
+      float v = acc[m][c];
+#pragma unroll
+      for (int o = TK_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TK_WAVE);
+      if (lane == 0 && n0 + c < N) {
+        if (residual) v = round_to<T>(v) + to_f32<T>(residual[(size_t)(m0 + m) * ldr + n0 + c]);
+        C[(size_t)(m0 + m) * ldc + n0 + c] = from_f32<TO>(v);
+      }
+    }
+  }
+}
+
+template <typename T, typename TO>
+static void launch_rows(const T* A, int lda, const T* W, TO* C, int ldc, const T* residual, int ldr, int M,
+                        int N, int K, hipStream_t stream) {
+  const bool vec = sizeof(T) == 4 && K % 4 == 0 && lda % 4 == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
+  const int cols_per_block = (256 / TK_WAVE) * GR_COLS;
+  const unsigned gx = (unsigned)((N + cols_per_block - 1) / cols_per_block);
+#define TK_ROWS_LAUNCH(MB, VEC)                                                                        \
+  hipLaunchKernelGGL((gemm_rows_kernel<T, TO, MB, VEC>), dim3(gx, (M + MB - 1) / MB), dim3(256), 0, stream, \
+                     A, lda, W, C, ldc, residual, ldr, M, N, K)
+  if (M <= 4) {
+    if (vec) TK_ROWS_LAUNCH(4, true); else TK_ROWS_LAUNCH(4, false);
+  } else {
+    if (vec) TK_ROWS_LAUNCH(16, true); else TK_ROWS_LAUNCH(16, false);
+  }
+#undef TK_ROWS_LAUNCH
+}
 
 #define GT_BM 64
 #define GT_BN 64
@@ -76,6 +160,16 @@ TK_API int tk_gemm_generic(int dt, const void* A, int lda, const void* W, void* 
              M, N, K, lda, ldc);
   TK_REQUIRE(!residual || ldr >= N, "gemm_generic: residual stride %d < N %d", ldr, N);
   if (M == 0) return 0;
+  if (M <= GR_MAX_ROWS) {
+    if (dt == TK_F32)
+      launch_rows<float, float>((const float*)A, lda, (const float*)W, (float*)C, ldc, (const float*)residual, ldr, M, N, K, stream);
+    else if (out_f32)
+      launch_rows<bf16_t, float>((const bf16_t*)A, lda, (const bf16_t*)W, (float*)C, ldc, (const bf16_t*)residual, ldr, M, N, K, stream);
+    else
+      launch_rows<bf16_t, bf16_t>((const bf16_t*)A, lda, (const bf16_t*)W, (bf16_t*)C, ldc, (const bf16_t*)residual, ldr, M, N, K, stream);
+    TK_CHECK_LAUNCH("gemm_rows");
+    return 0;
+  }
   dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM);
   TK_REQUIRE(grid.y < 65536, "gemm_generic: M=%d needs too many row tiles", M);
   if (dt == TK_F32) {
