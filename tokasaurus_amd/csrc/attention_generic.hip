@@ -8,8 +8,8 @@
 // only on the token's own position, never on the batch), and keeps a running
 // maximum, sum and weighted value sum per query head (online softmax).
 //
-//   K pages: [page][kv head][P][d]      V pages: [page][kv head][d][P]
-//   block_table[req][pos / P] is the page of a position.
+//   K pages: [page][kv head][d / 8][P][8]   V pages: [page][kv head][P / 4][d][4]
+//   (key_offset and value_offset of common.h); block_table[req][pos / P] is the page of a position.
 // A query at position p sees positions max(0, p - window + 1) .. p (window <= 0: all).
 #include "common.h"
 
