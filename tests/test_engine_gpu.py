@@ -153,6 +153,8 @@ def recorded_against_eager(folder, page, cfg, live, lengths, max_tokens, budget=
         if graphs:
             sizes = {size for size, _ in engine.runner.recorded}
             assert sizes and all(step.captured for step in engine.runner.recorded.values())
+            # a recorded step carries table rows for its context bound, not for the longest request allowed
+            assert all(step.widths[0] <= -(-bound // page) for (_, bound), step in engine.runner.recorded.items())
         else:
             assert not any(step.captured for step in engine.runner.recorded.values())
     for (ta, la), (tb, lb) in zip(*results):

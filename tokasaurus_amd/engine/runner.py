@@ -129,7 +129,10 @@ class RecordedDecodeStep:
         self.model, self.storage, self.manager = model, storage, manager
         device = model.device
         B = size
-        widths = [t.shape[1] for t in manager.slot_tables]
+        # a table row as wide as the bound's pages, not as the longest request the engine allows
+        pages_in_bound = -(-kv_bound // runner.page_size)
+        widths = [min(t.shape[1], pages_in_bound) for t in manager.slot_tables]
+        self.widths = widths
         fields = [("token_ids", B), ("positions", B), ("token_req", B), ("q_start", B + 1), ("kv_len", B),
                   ("slots", B), ("token_slots", B), ("want_rows", B), ("temperature", B), ("uniform", B)]
         fields += [(f"table{g}", B * w) for g, w in enumerate(widths)]
@@ -228,7 +231,7 @@ class RecordedDecodeStep:
         rows = np.asarray(list(slots) + [self.null_slot] * pad, dtype=np.int64)
         for g, table in enumerate(self.manager.slot_tables):
             at, m = self.spans[f"table{g}"]
-            a[at : at + m].reshape(B, table.shape[1])[:] = table[rows]
+            a[at : at + m].reshape(B, self.widths[g])[:] = table[rows, : self.widths[g]]
 
     def run(self, planned: list[PlannedEntry], sampling: Sampling | None, write_slots: bool) -> StepOutput:
         n = len(planned)
