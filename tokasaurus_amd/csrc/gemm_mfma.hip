@@ -11,13 +11,15 @@
 // No workgroup talks to another and partial sums inside a workgroup are added in
 // wavefront order through LDS, so every output has one fixed order of summation.
 //
-// Two kernels:
-//   gemm_skinny_kernel (M <= 16, or any M as the fallback): a workgroup owns NT tiles
-//     and all of K; its wavefronts split K and read A straight from memory.
-//   gemm_staged_kernel (16 < M <= 128): a workgroup is 4 x WK wavefronts; the 4
-//     wavefronts of a row own NT tiles each and share the K range of their row, whose
-//     part of A passes through LDS (double buffered, 4 steps of 32 a round) so that A
-//     is read from the caches once per workgroup and not once per wavefront.
+// Two kernels (the entry point chooses; the engine calls it for up to 16 rows, for the
+// stacked q, k, v product up to 32):
+//   gemm_skinny_kernel: a workgroup owns NT tiles and all of K; its wavefronts split K
+//     and read A straight from memory.
+//   gemm_staged_kernel (a wide output, the head, from 5 rows on): a workgroup is
+//     4 x WK wavefronts; the 4 wavefronts of a row own NT tiles each and share the K
+//     range of their row, whose part of A passes through LDS (double buffered, 4 steps
+//     of 32 a round) so that A is read from the caches once per workgroup and not once
+//     per wavefront.
 //
 // Norm in front (sumsq_in != null).  The product of RMSNorm(x) is rstd[row] * ((x * w) W^T).
 // The kernel that produced x (the residual epilogue below, when emit_w is given) has
