@@ -96,7 +96,7 @@ def main(argv: list[str] | None = None) -> int:
     try:
         config = apply_overrides(RunConfig(), argv)
         return start(config)
-    except OptionError as e:
+    except ValueError as e:  # an option, or a request the engine refuses: say so without a traceback
         print(f"toka: {e}", file=sys.stderr)
         return 2
 
