@@ -353,3 +353,64 @@ def test_paced_prefill_changes_the_steps_and_no_completion(seed):
             assert cache.num_free_pages() == total and cache.slots.num_free == cache.slots.num_slots
             assert s.num_bumps == 0
     assert all(r == results[0] for r in results) and len(results[0]) > 0
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_workloads_with_aborts_windows_pacing_and_a_step_ahead(seed):
+    """Requests arrive, are aborted, end by length or at an end token, with one or two cache
+    groups (one windowed), reservation or optimistic admission, greedy or paced prompts, tokens
+    resolved at once or a step late: the cache manager's invariants hold after every step,
+    every request ends, and every page and slot comes back."""
+    rng = random.Random(seed)
+    P = rng.choice([2, 4, 16])
+    groups = [CacheGroup(CacheNeed(2, 16, 0), (0,))]
+    if rng.random() < 0.5:
+        groups.append(CacheGroup(CacheNeed(2, 16, rng.choice([3, 8, 20])), (1,)))
+    pages = rng.choice([16, 24, 40])
+    seqs = rng.choice([2, 4, 8])
+    cache = CacheManager(groups, pages, P, seqs)
+    s = Scheduler(cache, rng.choice([8, 24, 64]), seqs, max_num_tokens_per_request=10_000, eos_token_ids=(3,),
+                  optimistic=rng.random() < 0.5, max_prefill_chunk=rng.choice([None, 3]), sanity_checks=True,
+                  greedy_prefill=rng.random() < 0.5, prefill_round_up_multiple=rng.choice([1, 4, 16]))
+    submitted, finished, aborted = {}, {}, set()
+    inflight = None
+    nxt = 0
+    ahead = rng.random() < 0.5
+    for step in range(400):
+        if nxt < 30 and rng.random() < 0.4:
+            plen, mt = rng.randint(1, 20), rng.randint(1, 12)
+            if math.ceil((plen + mt - 1) / P) <= pages:
+                r = Request(f"r{nxt}", list(range(1, plen + 1)), SamplingParams(max_tokens=mt, ignore_eos=rng.random() < 0.3))
+                s.submit(r); submitted[r.id] = r
+            nxt += 1
+        if rng.random() < 0.08 and submitted:
+            rid = rng.choice(list(submitted))
+            if rid not in finished and rid not in aborted:
+                if s.abort(rid) is not None:
+                    aborted.add(rid)
+        d = s.schedule()
+        launched = None
+        if not d.empty():
+            toks = [random.Random(f"{seed}/{r.id}/{r.sampled}").choice([3, 5, 6, 7, 8]) for r in d.requests_with_output()]
+            s.advance(d); launched = (d, toks)
+        if inflight is not None:
+            for r in s.resolve(inflight[0], inflight[1], None): finished[r.id] = r
+            inflight = None
+        if launched is not None:
+            if ahead: inflight = launched
+            else:
+                for r in s.resolve(launched[0], launched[1], None): finished[r.id] = r
+        cache.check()
+        if nxt >= 30 and not s.has_work() and inflight is None:
+            break
+    assert not s.has_work(), (seed, "work left", len(s.queued), len(s.prefilling), len(s.decoding))
+    for rid, r in submitted.items():
+        assert rid in finished or rid in aborted, (seed, rid, r.state, r.finish_reason)
+    assert cache.num_free_pages() == [pages] * len(groups), (seed, cache.num_free_pages())
+    assert cache.slots.num_free == cache.slots.num_slots
+    for rid, r in finished.items():
+        if rid in aborted: continue
+        assert 1 <= len(r.completion) <= r.params.max_tokens
+        assert r.finish_reason in ("length", "stop")
+        if r.finish_reason == "length": assert len(r.completion) == r.params.max_tokens
+        else: assert r.completion[-1] == 3 and 3 not in r.completion[:-1]
