@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import plain_llama
+import toy_parts
 from gpu_common import TOL, plain_generate
 from replay_helpers import compare, compare_with_bfloat16_measure, mixed_trace, plain_rows, run_steps
 from tiny_models import make_folder, random_tokens
@@ -108,3 +109,46 @@ def test_generation_under_random_options(tmp_path, seed):
         if c.topk_ids is not None:
             assert [len(t) for t in c.topk_ids] == [2] * len(c.tokens)
     assert engine.runner.manager.num_free_pages() == [p.num_pages for p in engine.runner.manager.pools]
+
+
+@pytest.mark.parametrize("seed", [0, 3, 7, 12, 21, 22])
+def test_a_random_arrangement_of_layers(tmp_path, seed):
+    """A random configuration whose run order is drawn at random too: two to five entries that
+    name layers in any order and more than once, some reading the cache of an earlier entry,
+    some layers with a sliding window (5, 17 or 40 keys): mixed batches on few pages against the
+    plain implementation run in the same arrangement."""
+    toy_parts.register()
+    rng = random.Random(seed)
+    cfg = random_config(rng)
+    layers = rng.choice([2, 3])
+    cfg["num_hidden_layers"] = layers
+    windows = {str(i): rng.choice([5, 17, 40]) for i in range(layers) if rng.random() < 0.4}
+    order: list[list] = []
+    for place in range(rng.randint(2, 5)):
+        layer, source = rng.randrange(layers), None
+        if place > 0 and rng.random() < 0.35:
+            # an entry may read the cache of an earlier entry that keeps one and sees as far back
+            fits = [j for j, (lj, sj) in enumerate(order) if sj is None and windows.get(str(lj)) == windows.get(str(layer))]
+            if fits:
+                source = rng.choice(fits)
+        order.append([layer, source])
+    cfg.update(model_type="toy_arranged", toy_run_order=order, toy_windows=windows)
+    page = rng.choice([4, 8, 16, 32])
+    folder = make_folder(tmp_path / "m", cfg, seed=seed)
+    lengths = [rng.randint(1, 160) for _ in range(rng.randint(3, 6))]
+    print(f"seed {seed}: page {page}, lengths {lengths}, {cfg}")
+    requests = {f"r{i}": random_tokens(n, cfg["vocab_size"], 1000 * seed + i) for i, n in enumerate(lengths)}
+    pcfg, w = plain_llama.load_folder(folder)
+    plain = {rid: toy_parts.plain_arranged_logits(pcfg, w, toks) for rid, toks in requests.items()}
+    cfg16, w16 = plain_llama.load_folder(folder, torch.bfloat16)
+    plain16 = {rid: toy_parts.plain_arranged_logits(cfg16, w16, toks) for rid, toks in requests.items()}
+    tokens = sum(sorted(-(-n // 64) * 64 for n in lengths)[-4:])
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner.from_folder(folder, dtype, page_size=page, num_pages=-(-tokens // page), max_slots=4)
+        got = run_steps(runner, mixed_trace(requests, seed=seed))
+        assert len(got) == sum(lengths)
+        if dtype == "float32":
+            compare(got, plain, **TOL[dtype])
+        else:
+            compare_with_bfloat16_measure(got, plain, plain16, **TOL[dtype])
+        assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
