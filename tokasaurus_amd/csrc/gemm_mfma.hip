@@ -640,7 +640,7 @@ struct GemmExtra {
 // Number of partial sums a row gets from the residual epilogue with emit_w: one a tile.
 TK_API int tk_gemm_skinny_parts(int M, int N, int tile_rows) {
   const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
-  const int th = tile_rows > 0 ? tile_rows : ((MB == 1 && (N + 15) / 16 < 256) ? 8 : 16);
+  const int th = tile_rows > 0 ? tile_rows : ((MB <= 2 && (N + 15) / 16 < 256) ? 8 : 16);
   return (N + th - 1) / th;
 }
 
@@ -727,7 +727,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
     }
   } else {
     // fewer tiles than compute units: tiles of 8 rows make twice the workgroups
-    a.TH = tile_rows > 0 ? tile_rows : ((MB == 1 && n16 < 256) ? 8 : 16);
+    a.TH = tile_rows > 0 ? tile_rows : ((MB <= 2 && n16 < 256) ? 8 : 16);
     const int th_units = (N + a.TH - 1) / a.TH;
     int groups;
     if (epi == EPI_ROPE) {
