@@ -638,9 +638,39 @@ struct GemmExtra {
 };
 
 // Number of partial sums a row gets from the residual epilogue with emit_w: one a tile.
+// Compute units of the current device (the workgroups that run at a time, one each).
+static int compute_units() {
+  static int units = 0;
+  if (units == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      units = n;
+    else
+      units = 256;
+  }
+  return units;
+}
+
+// Weight rows of a tile that the skinny kernel uses for up to 32 rows of A: 16 fill the matrix
+// core, fewer make more workgroups.  A workgroup streams its rows over all of K, so the time is
+// that of the rounds of workgroups the compute units take, times the rows of each: the fewest
+// win, and among equals the larger tile (A is read once a workgroup).
+// With the rotation epilogue (heads > 0) a workgroup takes `th` columns of one half of a head.
+static int choose_tile_rows(int M, int N, int heads = 0, int half = 0) {
+  if (M > 32) return 16;
+  const int units = compute_units();
+  int best = 16, best_cost = 0;
+  for (int th = 16; th >= 8; th -= 4) {
+    const int groups = heads > 0 ? heads * ((half + th - 1) / th) : (N + th - 1) / th;
+    const int cost = ((groups + units - 1) / units) * th;
+    if (th == 16 || cost < best_cost) { best = th; best_cost = cost; }
+  }
+  return best;
+}
+
 TK_API int tk_gemm_skinny_parts(int M, int N, int tile_rows) {
-  const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8));
-  const int th = tile_rows > 0 ? tile_rows : ((MB <= 2 && (N + 15) / 16 < 256) ? 8 : 16);
+  const int th = tile_rows > 0 ? tile_rows : choose_tile_rows(M, N);
   return (N + th - 1) / th;
 }
 
@@ -664,7 +694,7 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
              "gemm_skinny: rows of A and W must be 16-byte aligned (lda=%d)", lda);
   TK_REQUIRE(lda >= K, "gemm_skinny: lda %d shorter than K %d", lda, K);
   TK_REQUIRE(epi != EPI_RESIDUAL || (residual && ldr >= N), "gemm_skinny: residual missing or too narrow");
-  TK_REQUIRE(tile_rows == 0 || tile_rows == 4 || tile_rows == 8 || tile_rows == 16, "gemm_skinny: tile_rows %d is not 0, 4, 8 or 16", tile_rows);
+  TK_REQUIRE(tile_rows == 0 || tile_rows == 4 || tile_rows == 8 || tile_rows == 12 || tile_rows == 16, "gemm_skinny: tile_rows %d is not 0, 4, 8, 12 or 16", tile_rows);
   if (M == 0) return 0;
   GemmArgs a = {};
   a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.C = C; a.ldc = ldc;
@@ -726,8 +756,8 @@ TK_API int tk_gemm_skinny_bf16(const void* A, int lda, const void* W, void* C, i
       default: ok = launch_mb<8, true>(a, epi, norm, NT, groups, WK, stream); break;
     }
   } else {
-    // fewer tiles than compute units: tiles of 8 rows make twice the workgroups
-    a.TH = tile_rows > 0 ? tile_rows : ((MB <= 2 && n16 < 256) ? 8 : 16);
+    a.TH = tile_rows > 0 ? tile_rows
+                         : (epi == EPI_ROPE ? choose_tile_rows(M, N, a.nq + 2 * a.nkv, a.d / 2) : choose_tile_rows(M, N));
     const int th_units = (N + a.TH - 1) / a.TH;
     int groups;
     if (epi == EPI_ROPE) {

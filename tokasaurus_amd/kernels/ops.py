@@ -597,8 +597,8 @@ SKINNY_MAX_ROWS = 128  # rows the weight-streaming kernel takes
 # 1B model, whole recorded decode steps at a context of 1,024: at 8 and 16 rows 19 and 11 %
 # faster than the library product followed by the kernels it fuses away (rotation and append,
 # SwiGLU, norms); at 24 and 32 rows 12 % slower, at 64 rows a third.  At the wider 3B and 8B
-# shapes it is ahead up to 8 rows (at one row by 14 and 21 %); at 16 rows the library is, by 13
-# and 1 %: its long products (the down projection) are then short of workgroups to balance.
+# shapes it is ahead up to 8 rows (at one row by 21 %, at 8 rows by 10 %) and level with the
+# library at 16.
 SKINNY_ROWS = 16
 # The stacked q, k, v product with rotation and append in its epilogue replaces two kernels of
 # the library path and has a short inner size: it stays ahead up to 32 rows (4 % of a step).
