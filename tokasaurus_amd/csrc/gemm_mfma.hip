@@ -655,7 +655,8 @@ static int compute_units() {
 // Weight rows of a tile that the skinny kernel uses for up to 32 rows of A: 16 fill the matrix
 // core, fewer make more workgroups.  A workgroup streams its rows over all of K, so the time is
 // that of the rounds of workgroups the compute units take, times the rows of each: the fewest
-// win, and among equals the larger tile (A is read once a workgroup).
+// win, and among equals the larger tile (A is read once a workgroup).  With two rounds or more
+// of full tiles the rounds overlap and even out: 16 rows then (measured: smaller tiles lose).
 // With the rotation epilogue (heads > 0) a workgroup takes `th` columns of one half of a head.
 static int choose_tile_rows(int M, int N, int heads = 0, int half = 0) {
   if (M > 32) return 16;
@@ -663,6 +664,7 @@ static int choose_tile_rows(int M, int N, int heads = 0, int half = 0) {
   int best = 16, best_cost = 0;
   for (int th = 16; th >= 8; th -= 4) {
     const int groups = heads > 0 ? heads * ((half + th - 1) / th) : (N + th - 1) / th;
+    if (th == 16 && groups >= 2 * units) return 16;
     const int cost = ((groups + units - 1) / units) * th;
     if (th == 16 || cost < best_cost) { best = th; best_cost = cost; }
   }
