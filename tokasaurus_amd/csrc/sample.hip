@@ -11,6 +11,9 @@
 //   sample_finish:  one workgroup per row: joins the chunks in chunk order, finds
 //                   the chunk in which the cumulative mass passes u, and scans it.
 #include "common.h"
+#include "sample.h"
+
+#include <mutex>
 
 #define SM_THREADS 256
 #define SM_PER_THREAD 8
@@ -173,6 +176,21 @@ __global__ __launch_bounds__(SM_THREADS) void sample_finish_kernel(
 
 TK_API int tk_sample_chunks(int vocab) { return (vocab + SM_CHUNK - 1) / SM_CHUNK; }
 
+// The two launches of the sampler on checked arguments.
+static int launch_sample(const float* logits, int ld, int rows, int vocab, const float* temperature,
+                         const float* uniform, const int* slots, int* last_token, int* out_ids,
+                         float* out_logprobs, float* part_max, float* part_sum, int* part_arg,
+                         int n_chunks, hipStream_t stream) {
+  hipLaunchKernelGGL(sample_partial_kernel, dim3(n_chunks, rows), dim3(SM_THREADS), 0, stream, logits,
+                     ld, vocab, temperature, part_max, part_sum, part_arg, n_chunks);
+  TK_CHECK_LAUNCH("sample_partial");
+  hipLaunchKernelGGL(sample_finish_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, vocab,
+                     temperature, uniform, part_max, part_sum, part_arg, n_chunks, slots, last_token,
+                     out_ids, out_logprobs);
+  TK_CHECK_LAUNCH("sample_finish");
+  return 0;
+}
+
 // part_max, part_sum (float) and part_arg (int) hold rows * tk_sample_chunks(vocab) entries each.
 TK_API int tk_sample(const float* logits, int ld, int rows, int vocab, const float* temperature,
                          const float* uniform, const int* slots, int* last_token, int* out_ids,
@@ -186,14 +204,62 @@ TK_API int tk_sample(const float* logits, int ld, int rows, int vocab, const flo
   TK_REQUIRE(rows < 65536, "sample: %d rows are too many for one call", rows);
   TK_REQUIRE(part_max && part_sum && part_arg, "sample: scratch missing");
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(sample_partial_kernel, dim3(n_chunks, rows), dim3(SM_THREADS), 0, stream, logits,
-                     ld, vocab, temperature, part_max, part_sum, part_arg, n_chunks);
-  TK_CHECK_LAUNCH("sample_partial");
-  hipLaunchKernelGGL(sample_finish_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, vocab,
-                     temperature, uniform, part_max, part_sum, part_arg, n_chunks, slots, last_token,
-                     out_ids, out_logprobs);
-  TK_CHECK_LAUNCH("sample_finish");
-  return 0;
+  return launch_sample(logits, ld, rows, vocab, temperature, uniform, slots, last_token, out_ids, out_logprobs,
+                       part_max, part_sum, part_arg, n_chunks, stream);
+}
+
+// ---------------------------------------------------------------------------
+// tk_sample_static: the partial results in a device array of the library's own (sample.h).
+// In host code the array's name is only a handle: its address on a GPU comes from
+// hipGetSymbolAddress, asked once per device with that device current (every GPU has a copy
+// of the array at an address of its own), and only that address is given to kernels.
+#define SAMPLE_STATIC_DEVICES 64
+static __device__ __align__(256) uint32_t scratch[3 * TK_SAMPLE_STATIC_ITEMS];
+static void* g_scratch_ptr[SAMPLE_STATIC_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// The array's address on the current device (null, with the error text set, on failure).
+static uint32_t* static_scratch() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= SAMPLE_STATIC_DEVICES) {
+    tk_set_error("sample_static: no usable current device (%s, device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      tk_set_error("sample_static: the scratch array has no address on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return (uint32_t*)g_scratch_ptr[dev];
+}
+
+TK_API int tk_sample_static(const float* logits, int ld, int rows, int vocab, const float* temperature,
+                            const float* uniform, const int* slots, int* last_token, int* out_ids,
+                            float* out_logprobs, hipStream_t stream) {
+  TK_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "sample_static: bad sizes rows=%d vocab=%d ld=%d", rows,
+             vocab, ld);
+  const int n_chunks = (vocab + SM_CHUNK - 1) / SM_CHUNK;
+  TK_REQUIRE(n_chunks <= SM_MAX_CHUNKS, "sample_static: a vocabulary of %d is larger than %d", vocab,
+             SM_MAX_CHUNKS * SM_CHUNK);
+  TK_REQUIRE((long)rows * n_chunks <= TK_SAMPLE_STATIC_ITEMS,
+             "sample_static: %d rows of %d chunks need %ld partial results, the static scratch holds %d; "
+             "use tk_sample with a workspace for inputs this large",
+             rows, n_chunks, (long)rows * n_chunks, TK_SAMPLE_STATIC_ITEMS);
+  if (rows == 0) return 0;
+  uint32_t* base = static_scratch();
+  if (base == nullptr) return -3;
+  // every (row, chunk) entry that the second kernel reads is written by the first: nothing to clear
+  float* part_max = (float*)base;
+  float* part_sum = (float*)(base + TK_SAMPLE_STATIC_ITEMS);
+  int* part_arg = (int*)(base + 2 * TK_SAMPLE_STATIC_ITEMS);
+  return launch_sample(logits, ld, rows, vocab, temperature, uniform, slots, last_token, out_ids, out_logprobs,
+                       part_max, part_sum, part_arg, n_chunks, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -36,6 +36,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         + [c_float, _P],
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
         "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
+        "tk_sample_static": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_chunks": [c_int],
         "tk_topk_logprobs": [_P, c_int, c_int, c_int, _P, c_int, _P, _P, _P, _P, _P, _P, _P],
     },
