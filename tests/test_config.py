@@ -58,6 +58,11 @@ def test_registry_picks_by_model_type_and_lists_known_names():
         architecture_of({"model_type": "mamba"})
     with pytest.raises(ConfigError, match="model_type"):
         architecture_of({})
+    # a file without model_type is taken by the class name it gives under "architectures"
+    no_type = {k: v for k, v in CONFIG_A.items() if k != "model_type"}
+    assert architecture_of(dict(no_type, architectures=["LlamaForCausalLM"])).name == "llama"
+    with pytest.raises(ConfigError, match="LlamaForCausalLM"):
+        architecture_of(dict(no_type, architectures=["SomethingElse"]))
 
 
 def test_model_is_built_from_the_config_alone():

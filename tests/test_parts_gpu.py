@@ -214,6 +214,64 @@ def all_cuttings(runner, reqs, ref, tol):
     assert all(pool.num_free == pool.num_pages for pool in runner.manager.pools)
 
 
+def test_a_model_of_state_mixers_alone_generates_through_the_engine(tmp_path):
+    """Every layer's mixer is the toy recurrence and the embedding is the toy's scaled one: the
+    model has no cache group at all.  It is registered from the tests, scheduled, stepped
+    (recorded decode steps included) and sampled through the engine without a change to the
+    framework, more requests than slots, so that slots are reused: a request that takes a
+    used slot must start from zeroed state."""
+    from tokasaurus_amd import EngineConfig, SamplingParams
+    from tokasaurus_amd.engine.engine import Engine
+
+    toy_parts.register()
+    config = dict(CONFIG_A, model_type="toy_recurrent", num_hidden_layers=2, toy_state_size=24, toy_recurrent_layers=[0, 1],
+                  toy_embedding_scale=1.5)
+    folder = write_random_model(tmp_path / "toy", config, seed=6)
+    sharpen(folder, {"mixer.in.weight": 5.0, "mixer.out.weight": 5.0})
+    cfg, w = plain_llama.load_folder(folder)
+    prompts = [random_tokens(n, cfg["vocab_size"], 70 + n) for n in (7, 19, 3, 12, 26, 5)]
+
+    def plain_greedy(prompt, n, config=cfg):
+        ids, out = list(prompt), []
+        for _ in range(n):
+            out.append(int(toy_parts.plain_toy_recurrent_logits(config, w, ids)[-1].argmax()))
+            ids.append(out[-1])
+        return out
+
+    # the embedding's scale matters to the tokens: a model that ignored it would be found out
+    assert any(plain_greedy(p, 6) != plain_greedy(p, 6, dict(cfg, toy_embedding_scale=None)) for p in prompts)
+    engine = Engine(EngineConfig(model=str(folder), dtype="float32", page_size=4, kv_cache_num_tokens=64, max_seqs_per_forward=2,
+                                 max_tokens_per_forward=16, allocator_sanity_checks=True))
+    assert engine.runner.groups == [] and engine.runner.manager.pools == []
+    done = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
+    for prompt, c in zip(prompts, done):
+        assert c.tokens == plain_greedy(prompt, 6), c.request_id
+    assert engine.runner.recorded, "decode steps of the toy model were not recorded"
+    assert engine.runner.manager.slots.num_free == 2
+
+
+def test_a_request_that_takes_a_used_slot_starts_from_zeroed_state(tmp_path):
+    """One slot: the second request gets the slot the first one left its state in, and its
+    logits equal those of a fresh runner (and of the plain model)."""
+    toy_parts.register()
+    config = dict(CONFIG_A, model_type="toy_recurrent", num_hidden_layers=3, toy_state_size=24, toy_recurrent_layers=[1])
+    folder = write_random_model(tmp_path / "toy", config, seed=4)
+    sharpen(folder, {"mixer.in.weight": 5.0, "mixer.out.weight": 5.0})
+    cfg, w = plain_llama.load_folder(folder)
+    first, second = random_tokens(30, cfg["vocab_size"], 1), random_tokens(21, cfg["vocab_size"], 2)
+    ref = {"second": toy_parts.plain_toy_recurrent_logits(cfg, w, second)}
+    used = ModelRunner.from_folder(folder, "float32", page_size=4, num_pages=32, max_slots=1)
+    run_steps(used, whole("first", first))
+    assert used.storage.states[1].abs().max() > 0  # the first request left its state behind
+    # decoded one by one from the start: position 0 runs as a recorded one-token step
+    got_used = run_steps(used, tail_one_by_one("second", second, len(second) - 1))
+    fresh = ModelRunner.from_folder(folder, "float32", page_size=4, num_pages=32, max_slots=1)
+    got_fresh = run_steps(fresh, tail_one_by_one("second", second, len(second) - 1))
+    compare(got_used, ref, **TOL["float32"])
+    for key, row in got_fresh.items():
+        assert torch.equal(row, got_used[key]), key
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_mixer_with_state_of_its_own(tmp_path, dtype):
     """A toy recurrent mixer, defined in the tests, is registered, built from a

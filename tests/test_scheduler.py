@@ -414,3 +414,41 @@ def test_random_workloads_with_aborts_windows_pacing_and_a_step_ahead(seed):
         assert r.finish_reason in ("length", "stop")
         if r.finish_reason == "length": assert len(r.completion) == r.params.max_tokens
         else: assert r.completion[-1] == 3 and 3 not in r.completion[:-1]
+
+
+@pytest.mark.parametrize("greedy", [True, False])
+def test_a_model_without_any_cache_group_is_scheduled(greedy):
+    """Every mixer keeps state of fixed size: no pages exist, so none can run out; slots and
+    the token budget are the only limits (admission, pacing and decoding all pass through
+    the page arithmetic)."""
+    cache = CacheManager([], 8, 4, 3)
+    s = Scheduler(cache, max_tokens_per_forward=16, max_seqs_per_forward=3, max_num_tokens_per_request=1000,
+                  sanity_checks=True, greedy_prefill=greedy, prefill_round_up_multiple=4)
+    for i, (n, m) in enumerate([(20, 3), (5, 4), (9, 2), (7, 5), (30, 1)]):
+        s.submit(req(f"r{i}", n, m))
+    done, steps = [], 0
+    while s.has_work():
+        d, fin = run_step(s)
+        assert not d.empty() and d.num_tokens() <= 16
+        assert len(s.running()) <= 3
+        done += fin
+        steps += 1
+        assert steps < 200
+    assert sorted(r.id for r in done) == [f"r{i}" for i in range(5)]
+    assert all(len(r.completion) == r.params.max_tokens for r in done)
+    assert cache.slots.num_free == 3 and not cache.requests
+
+
+def test_fresh_slots_are_reported_once():
+    """A slot handed to a request is named exactly once, so that per-slot state is cleared
+    once, before the request's first step: also when the slot is reused, and after a bump."""
+    s, cache = make(num_pages=64, max_seqs=2, slots=2)
+    s.submit(req("a", 5, 2))
+    s.submit(req("b", 5, 2))
+    s.submit(req("c", 5, 2))
+    run_step(s)
+    assert sorted(cache.take_fresh_slots()) == [0, 1] and cache.take_fresh_slots() == []
+    while s.has_work():
+        run_step(s)
+    reused = cache.take_fresh_slots()
+    assert len(reused) == 1 and reused[0] in (0, 1)  # c took a slot that a or b gave back

@@ -21,6 +21,8 @@ from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.models import Architecture, ModelSpec, RunEntry, register_architecture
 from tokasaurus_amd.models.llama import llama_spec
 from tokasaurus_amd.parts.base import (
+    EMBEDDINGS,
+    Embedding,
     FEED_FORWARDS,
     INT_TABLE,
     MIXERS,
@@ -43,7 +45,7 @@ from tokasaurus_amd.parts.linear import Linear
 @MIXERS.register("toy_recurrence", replace=True)
 class ToyRecurrence(Mixer):
     """Keeps one vector of ``state_size`` 32-bit numbers per request, in the
-    request's slot.  A request's state starts from zero at position 0."""
+    request's slot, which the framework zeroes when a request takes it."""
 
     def __init__(self, hidden_size: int, state_size: int, names: dict[str, str]):
         self.hidden_size, self.state_size = hidden_size, state_size
@@ -70,15 +72,13 @@ class ToyRecurrence(Mixer):
             # one token a request: device arrays only, so the step can be recorded and replayed
             slots = ctx.slots.long()
             prev = state.index_select(0, slots)
-            prev = torch.where((ctx.positions == 0)[:, None], torch.zeros_like(prev), prev)
             s_all = self.decay[None, :] * prev + u
             state.index_copy_(0, slots, s_all)
         else:
             s_all = torch.empty_like(u)
             for r in range(ctx.num_requests):
                 a, b = ctx.host_q_start[r], ctx.host_q_start[r + 1]
-                start = ctx.host_kv_len[r] - (b - a)
-                s = state[ctx.host_slots[r]].clone() if start > 0 else torch.zeros_like(state[0])
+                s = state[ctx.host_slots[r]].clone()
                 for t in range(a, b):
                     s = self.decay * s + u[t]
                     s_all[t] = s
@@ -100,15 +100,38 @@ def plain_recurrence(h: torch.Tensor, w: dict, prefix: str) -> torch.Tensor:
     return torch.stack(out)
 
 
+@EMBEDDINGS.register("toy_scaled_embedding", replace=True)
+class ToyScaledEmbedding(Embedding):
+    """A row gather times a constant: an embedding of another kind than the framework's,
+    chosen by the model's specification alone."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, scale: float):
+        self.vocab_size, self.hidden_size, self.name, self.scale = vocab_size, hidden_size, name, float(scale)
+        self.table: torch.Tensor | None = None
+
+    def tensor_specs(self) -> list[TensorSpec]:
+        return [TensorSpec(self.name, (self.vocab_size, self.hidden_size))]
+
+    def load(self, tensors, placer) -> None:
+        self.table = placer.place(("row_major", self.name), lambda: tensors[self.name].to(placer.dtype).contiguous().to(placer.device))
+
+    def forward(self, ctx):
+        x = ops.embed_gather(ctx.token_ids, self.table, ctx.last_token)
+        return (x.float() * self.scale).to(x.dtype)
+
+
 @dataclass(frozen=True)
 class ToyConfig:
     llama: LlamaConfig
     state_size: int
     recurrent_layers: tuple[int, ...]
+    embedding_scale: float | None = None
 
     @staticmethod
     def from_dict(d: dict[str, Any]) -> "ToyConfig":
-        return ToyConfig(LlamaConfig.from_dict(d), int(d["toy_state_size"]), tuple(d["toy_recurrent_layers"]))
+        scale = d.get("toy_embedding_scale")
+        return ToyConfig(LlamaConfig.from_dict(d), int(d["toy_state_size"]), tuple(d["toy_recurrent_layers"]),
+                         None if scale is None else float(scale))
 
 
 def toy_recurrent_spec(cfg: ToyConfig) -> ModelSpec:
@@ -123,12 +146,15 @@ def toy_recurrent_spec(cfg: ToyConfig) -> ModelSpec:
              "names": {"in": f"{p}.mixer.in.weight", "out": f"{p}.mixer.out.weight", "decay": f"{p}.mixer.decay"}},
         )
         layers[i] = PartSpec(layers[i].kind, params)
-    return ModelSpec(**{**base.__dict__, "layers": tuple(layers)})
+    fields = {**base.__dict__, "layers": tuple(layers)}
+    if cfg.embedding_scale is not None:
+        fields["embedding"] = PartSpec("toy_scaled_embedding", {**base.embedding.params, "scale": cfg.embedding_scale})
+    return ModelSpec(**fields)
 
 
 def plain_toy_recurrent_logits(cfg: dict, w: dict, token_ids: list[int]) -> torch.Tensor:
     d = cfg["hidden_size"] // cfg["num_attention_heads"]
-    x = w["model.embed_tokens.weight"][torch.tensor(token_ids)]
+    x = w["model.embed_tokens.weight"][torch.tensor(token_ids)] * float(cfg.get("toy_embedding_scale") or 1.0)
     inv = plain_llama.rope_inverse_frequencies(d, float(cfg["rope_theta"]), cfg.get("rope_scaling"))
     cos, sin = plain_llama.rope_tables(torch.arange(len(token_ids)), inv)
     for i in range(cfg["num_hidden_layers"]):

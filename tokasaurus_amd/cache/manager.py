@@ -88,6 +88,9 @@ class CacheManager:
         self.pools = [PagePool(n) for n in counts]
         self.slots = SlotAllocator(max_slots)
         self.requests: dict[str, RequestCache] = {}
+        # slots handed out since the owner of the state tensors last asked: a request must
+        # not inherit the state that the slot's last holder left
+        self.fresh_slots: list[int] = []
         # Per group, the block tables once more as one array indexed by slot, kept
         # up to date as pages come and go: a step whose shape is fixed (a recorded
         # decode step) gathers its rows from it instead of walking lists.  Row
@@ -120,9 +123,16 @@ class CacheManager:
         if request_id in self.requests:
             raise ValueError(f"request {request_id!r} is already live")
         slot = self.slots.allocate()
+        self.fresh_slots.append(slot)
         rc = RequestCache(request_id, slot, [[] for _ in self.groups], first_held=[0] * len(self.groups))
         self.requests[request_id] = rc
         return rc
+
+    def take_fresh_slots(self) -> list[int]:
+        """The slots given to requests since the last call (each once): whoever owns
+        per-slot state clears it for them before their first step."""
+        out, self.fresh_slots = self.fresh_slots, []
+        return out
 
     def reserve(self, request_id: str, new_len: int) -> None:
         """Make room for the request to hold ``new_len`` tokens in every group,

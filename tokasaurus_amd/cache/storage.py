@@ -46,5 +46,15 @@ class CacheStorage:
         # slot `max_slots` belongs to no request (padding rows of a recorded step use it)
         self.last_token = torch.zeros((max_slots + 1,), dtype=torch.int32, device=device)
 
+    def reset_slots(self, slots: list[int]) -> None:
+        """Zero the state of these slots in every state tensor: a request that takes a slot
+        starts from the state a fresh engine would give it, whoever held the slot before."""
+        if not slots:
+            return
+        for t in self.states:
+            if t is not None:
+                for s in slots:
+                    t[s].zero_()
+
     def bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.keys + self.values)

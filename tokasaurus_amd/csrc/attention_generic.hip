@@ -139,6 +139,19 @@ static void ag_launch(const void* q, int q_stride, void* out, int out_stride, co
                      block_table, table_stride, token_req, positions, nq, nkv, d, P, window, scale);
 }
 
+// Whether the kernel takes this group and head size at all (0 and the reason in tk_last_error
+// when not): asked when a cache is made, so that a model is refused before its first step.
+TK_API int tk_paged_attention_generic_fits(int nq, int nkv, int d) {
+  TK_REQUIRE(nq > 0 && nkv > 0 && d > 0 && nq % nkv == 0, "paged_attention: bad sizes nq=%d nkv=%d d=%d", nq, nkv, d);
+  const int group = nq / nkv;
+  TK_REQUIRE(group * d <= AG_THREADS * AG_MAX_ACC,
+             "paged_attention: group %d x head size %d exceeds %d outputs per kv head", group, d,
+             AG_THREADS * AG_MAX_ACC);
+  TK_REQUIRE(ag_smem_bytes(group, d, 8) <= 64 * 1024,
+             "paged_attention: head size %d with group %d does not fit the local memory", d, group);
+  return 0;
+}
+
 TK_API int tk_paged_attention_generic(int dt, const void* q, int q_stride, void* out,
                                           int out_stride, const void* kcache, const void* vcache,
                                           const int* block_table, int table_stride,

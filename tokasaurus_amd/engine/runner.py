@@ -281,6 +281,8 @@ class ModelRunner:
         if max_tokens_per_request is not None:
             limit = min(limit, max_tokens_per_request)
         self.max_tokens_per_request = limit
+        for block in model.blocks:  # a shape no attention kernel takes is refused here, not at the first step
+            block.mixer.check_cache(page_size, model.dtype)
         needs = model.cache_needs()
         cache_of = [e.cache_of for e in model.spec.run_order]
         self.groups, self.where = plan_groups(needs, cache_of)
@@ -333,9 +335,8 @@ class ModelRunner:
         arch, cfg = config_from_folder(model_dir, rope_scaling_override)
         model = build_model(arch, cfg)
         specs = model.tensor_specs()
-        # a checkpoint that ties its head may still carry the head's tensor
-        allow = ("lm_head.weight",) if model.spec.head_name == model.spec.embedding_name else ()
-        tensors = read_tensors(model_dir, specs, allow_unexpected=allow)
+        # a checkpoint that ties its head may still carry the head's tensor: read_tensors warns and goes on
+        tensors = read_tensors(model_dir, specs, allow_unexpected=model.spec.ignorable_tensors)
         model.load(tensors, DTYPES[dtype], device)
         return cls(model, page_size, num_pages, max_slots, **options)
 
@@ -412,6 +413,9 @@ class ModelRunner:
         entries and of their ``want`` lists; with ``sampling`` every wanted row is
         also sampled, and the token written to its request's slot."""
         planned = self.plan(entries)
+        # requests admitted since the last step (here or by a scheduler) start from zeroed state;
+        # in stream order before this step and after the last step of the slot's former holder
+        self.storage.reset_slots(self.manager.take_fresh_slots())
         write_slots = (sampling is not None) if write_slots is None else write_slots
         recorded = self._recorded_for(planned)
         if recorded is not None:

@@ -32,6 +32,7 @@ from tokasaurus_amd.cache.manager import CacheManager
 from tokasaurus_amd.sampling.params import SamplingParams
 
 QUEUED, PREFILLING, DECODING, FINISHED = "queued", "prefilling", "decoding", "finished"
+NO_PAGE_LIMIT = 1 << 60  # pages "free" when the model has no cache group at all
 
 
 @dataclass
@@ -146,7 +147,9 @@ class Scheduler:
 
     # ---- page arithmetic
     def _free_pages(self) -> int:
-        return min(self.cache.num_free_pages())
+        """Free pages of the scarcest group; a model without a cache group (every mixer keeps
+        state of fixed size) is never short of pages."""
+        return min(self.cache.num_free_pages(), default=NO_PAGE_LIMIT)
 
     def _held_blocks(self, req: Request) -> int:
         return len(self.cache.requests[req.id].tables[0]) if self.cache.groups else 0
@@ -211,7 +214,7 @@ class Scheduler:
             prompt_ends = -(-outstanding // self.last_num_prefill) - 1  # scheduler.py:73-86
             ends.append((prompt_ends + r.params.max_tokens - 1, r))
         ends.sort(key=lambda e: e[0])
-        total = min(pool.num_pages for pool in self.cache.pools)
+        total = min((pool.num_pages for pool in self.cache.pools), default=NO_PAGE_LIMIT)
         held = sum(pages.values())
         queued = list(self.queued.values())
         at, running = 0, len(ends)
@@ -244,7 +247,7 @@ class Scheduler:
         while True:
             need = 0
             for req in self.decoding.values():
-                need += max(self.cache.pages_needed(req.id, req.cache_tokens() + 1))
+                need += max(self.cache.pages_needed(req.id, req.cache_tokens() + 1), default=0)
             if need <= self._free_pages():
                 break
             victims = self.running()

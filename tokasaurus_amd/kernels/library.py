@@ -34,6 +34,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "tk_paged_attention_generic": [c_int, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P, _P]
         + [c_int] * 6
         + [c_float, _P],
+        "tk_paged_attention_generic_fits": [c_int, c_int, c_int],
         "tk_add": [c_int, _P, _P, _P, c_size_t, _P],
         "tk_sample": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P],
         "tk_sample_static": [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P],

@@ -340,6 +340,16 @@ def attention_mfma_supports(dtype: torch.dtype, head_dim: int, page_size: int) -
             and page_size >= 4 and page_size & (page_size - 1) == 0)
 
 
+def check_attention_shape(dtype: torch.dtype, nq: int, nkv: int, head_dim: int, page_size: int) -> None:
+    """Refuse, with the kernel's own reason, head counts and sizes that neither attention
+    kernel takes for this storage type and page size.  Called when a cache is made for a
+    mixer, so that a model that cannot run is refused before its first step."""
+    key_pages_shape(1, nkv, page_size, head_dim)
+    value_pages_shape(1, nkv, page_size, head_dim)
+    if not attention_mfma_supports(dtype, head_dim, page_size):
+        call("tk_paged_attention_generic_fits", nq, nkv, head_dim)
+
+
 def attention_tiles(
     q_lens: list[int], group: int, row_tiles: int, requests: list[int] | None = None, pair: bool = False
 ) -> tuple[list[int], list[int], list[int] | None]:

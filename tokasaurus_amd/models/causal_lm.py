@@ -8,9 +8,9 @@ import torch
 
 from tokasaurus_amd.kernels import ops
 from tokasaurus_amd.models.spec import ModelSpec
-from tokasaurus_amd.parts.base import BLOCKS, CacheNeed, CacheView, Part, StateNeed, StepContext, TensorSpec
+from tokasaurus_amd.parts.base import BLOCKS, EMBEDDINGS, HEADS, CacheNeed, CacheView, Part, StateNeed, StepContext, TensorSpec
 from tokasaurus_amd.parts.block import build_with_shared, stream_and_prepared
-from tokasaurus_amd.parts.embedding import LMHead, TokenEmbedding
+import tokasaurus_amd.parts.embedding  # noqa: F401  (registers the embedding and the head)
 from tokasaurus_amd.parts.linear import Placer
 
 
@@ -19,9 +19,9 @@ class CausalLM:
         spec.validate()
         self.spec = spec
         self.shared: dict = {}
-        self.embedding = TokenEmbedding(spec.vocab_size, spec.hidden_size, spec.embedding_name)
+        self.embedding = build_with_shared(EMBEDDINGS, spec.embedding, self.shared)
         self.blocks = [build_with_shared(BLOCKS, b, self.shared) for b in spec.layers]
-        self.head = LMHead(spec.vocab_size, spec.hidden_size, spec.head_name, spec.final_norm)
+        self.head = build_with_shared(HEADS, spec.head, self.shared)
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self.weight_bytes = 0
@@ -71,7 +71,7 @@ class CausalLM:
             rows = want_rows if i == last else None
             block = self.blocks[entry.layer]
             if block.fuses_norm:
-                next_norm = self.blocks[order[i + 1].layer].entry_norm() if i < last else self.head.norm
+                next_norm = self.blocks[order[i + 1].layer].entry_norm() if i < last else self.head.entry_norm()
                 out = block.forward(x, ctx, caches[i], states[i], rows, prepared=prepared, next_norm=next_norm)
             else:
                 out = block.forward(x, ctx, caches[i], states[i], rows)

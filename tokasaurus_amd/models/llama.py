@@ -66,12 +66,14 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
             )
         )
     embedding = "model.embed_tokens.weight"
+    final_norm = PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps, "name": "model.norm.weight"})
     return ModelSpec(
         vocab_size=cfg.vocab_size,
-        hidden_size=cfg.hidden_size,
-        embedding_name=embedding,
-        head_name=embedding if cfg.tie_word_embeddings else "lm_head.weight",
-        final_norm=PartSpec("rmsnorm", {"size": cfg.hidden_size, "eps": cfg.rms_norm_eps, "name": "model.norm.weight"}),
+        embedding=PartSpec("token_embedding", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size, "name": embedding}),
+        # a tied checkpoint's head names the embedding's tensor: both parts then share one buffer
+        head=PartSpec("norm_linear", {"vocab_size": cfg.vocab_size, "hidden_size": cfg.hidden_size, "norm": final_norm,
+                                      "name": embedding if cfg.tie_word_embeddings else "lm_head.weight"}),
+        ignorable_tensors=("lm_head.weight",) if cfg.tie_word_embeddings else (),
         layers=tuple(layers),
         run_order=tuple(RunEntry(i) for i in range(cfg.num_hidden_layers)),
         max_positions=cfg.max_position_embeddings,

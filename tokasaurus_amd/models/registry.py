@@ -20,6 +20,9 @@ class Architecture:
     name: str
     config_from_dict: Callable[[dict[str, Any]], Any]
     spec_from_config: Callable[[Any], ModelSpec]
+    # class names a config.json may give under "architectures" for this architecture: they
+    # choose it when the file has no model_type
+    class_names: tuple[str, ...] = ()
 
 
 ARCHITECTURES: dict[str, Architecture] = {}
@@ -31,13 +34,23 @@ def register_architecture(arch: Architecture, replace: bool = False) -> None:
     ARCHITECTURES[arch.name] = arch
 
 
-register_architecture(Architecture("llama", LlamaConfig.from_dict, llama_spec))
+register_architecture(Architecture("llama", LlamaConfig.from_dict, llama_spec, class_names=("LlamaForCausalLM",)))
 
 
 def architecture_of(config_dict: dict[str, Any]) -> Architecture:
+    """By ``model_type`` (the reference's only key, tokasaurus/model/utils.py:338-340); a file
+    without one is taken by the first name under ``architectures`` that a registered
+    architecture claims."""
     name = config_dict.get("model_type")
     if name is None:
-        raise ConfigError("config.json has no model_type")
+        classes = config_dict.get("architectures") or []
+        by_class = {c: a for a in ARCHITECTURES.values() for c in a.class_names}
+        for c in classes:
+            if c in by_class:
+                return by_class[c]
+        raise ConfigError(
+            f"config.json has no model_type and its architectures {list(classes)} name no registered model class; "
+            f"registered: model_type {sorted(ARCHITECTURES)}, architectures {sorted(by_class)}")
     if name not in ARCHITECTURES:
         raise ConfigError(f"unknown model_type {name!r}; registered architectures: {sorted(ARCHITECTURES)}")
     return ARCHITECTURES[name]

@@ -22,14 +22,15 @@ class RunEntry:
 @dataclass(frozen=True)
 class ModelSpec:
     vocab_size: int
-    hidden_size: int
-    embedding_name: str
-    head_name: str  # equals embedding_name when the checkpoint ties them
-    final_norm: PartSpec
+    embedding: PartSpec  # chosen from parts.base.EMBEDDINGS
+    head: PartSpec  # chosen from parts.base.HEADS (a head that names the embedding's tensor shares its buffer)
     layers: tuple[PartSpec, ...]  # block arrangements, each naming its own parts
     run_order: tuple[RunEntry, ...]
     max_positions: int
     eos_token_ids: tuple[int, ...] = ()
+    # tensors a checkpoint of this architecture may carry although the model reads them from
+    # elsewhere (the head's matrix of a checkpoint that ties it to the embedding)
+    ignorable_tensors: tuple[str, ...] = ()
 
     def validate(self) -> None:
         for i, e in enumerate(self.run_order):

@@ -4,6 +4,8 @@ built-in parts under their names."""
 from tokasaurus_amd.parts import attention, block, embedding, feedforward, norm, position  # noqa: F401
 from tokasaurus_amd.parts.base import (  # noqa: F401
     BLOCKS,
+    EMBEDDINGS,
+    HEADS,
     FEED_FORWARDS,
     MIXERS,
     NORMS,

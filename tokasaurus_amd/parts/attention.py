@@ -131,6 +131,9 @@ class PagedAttention(Mixer):
     def cache_need(self) -> CacheNeed:
         return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    def check_cache(self, page_size: int, dtype: torch.dtype) -> None:
+        ops.check_attention_shape(dtype, self.num_heads, self.num_kv_heads, self.head_dim, page_size)
+
     def load(self, tensors: dict[str, torch.Tensor], placer: Placer) -> None:
         self.qkv.load(tensors, placer)
         self.out.load(tensors, placer)

@@ -205,6 +205,10 @@ class Mixer(Part):
     def state_need(self) -> StateNeed | None:
         return None
 
+    def check_cache(self, page_size: int, dtype: torch.dtype) -> None:
+        """Called before the cache is made for this mixer: raise if its kernels do not take
+        pages of this size and storage type."""
+
     def forward(
         self,
         h: torch.Tensor,
@@ -223,6 +227,26 @@ class FeedForward(Part):
     fuses_norm = False
 
     def forward(self, h: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    """From the step's token ids to the first residual stream [N, H] in the engine dtype.
+    ``ctx.token_ids`` holds ids, or -(slot + 1) for a token to be read from ``ctx.last_token``."""
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """From the last residual stream (the wanted rows only) to logits [rows, vocab] in 32-bit.
+    ``entry_norm()`` is the norm it applies to its input first (or None): the last block may
+    prepare it, and hands what it prepared to ``forward`` as ``prepared``."""
+
+    def entry_norm(self) -> "Norm | None":
+        return None
+
+    def forward(self, x: torch.Tensor, prepared: "Prepared | None" = None) -> torch.Tensor:
         raise NotImplementedError
 
 
@@ -292,3 +316,5 @@ POSITION_ENCODINGS = Registry("position encoding")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block arrangement")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("head")

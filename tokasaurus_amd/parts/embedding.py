@@ -11,11 +11,13 @@ from __future__ import annotations
 import torch
 
 from tokasaurus_amd.kernels import ops
-from tokasaurus_amd.parts.base import MATRIX, NORMS, Normed, Part, PartSpec, Prepared, StepContext, TensorSpec
+from tokasaurus_amd.parts.base import (EMBEDDINGS, HEADS, MATRIX, NORMS, Embedding, Head, Normed, Part, PartSpec, Prepared,
+                                       StepContext, TensorSpec)
 from tokasaurus_amd.parts.linear import Linear, Placer
 
 
-class TokenEmbedding(Part):
+@EMBEDDINGS.register("token_embedding")
+class TokenEmbedding(Embedding):
     def __init__(self, vocab_size: int, hidden_size: int, name: str):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -35,7 +37,8 @@ class TokenEmbedding(Part):
         return ops.embed_gather(ctx.token_ids, self.table, ctx.last_token)
 
 
-class LMHead(Part):
+@HEADS.register("norm_linear")
+class LMHead(Head):
     def __init__(self, vocab_size: int, hidden_size: int, name: str, norm: PartSpec):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -44,6 +47,9 @@ class LMHead(Part):
 
     def children(self) -> list[Part]:
         return [self.norm]
+
+    def entry_norm(self):
+        return self.norm
 
     def tensor_specs(self) -> list[TensorSpec]:
         return self.norm.tensor_specs() + self.proj.tensor_specs()

@@ -16,6 +16,7 @@ its kernels, such as a matrix product, narrows it itself when it places it).
 from __future__ import annotations
 
 import json
+import logging
 from pathlib import Path
 
 import torch
@@ -25,6 +26,9 @@ from tokasaurus_amd.parts.base import INT_TABLE, TensorSpec
 
 SINGLE_FILE = "model.safetensors"
 INDEX_FILE = "model.safetensors.index.json"
+
+
+log = logging.getLogger("tokasaurus_amd")
 
 
 class WeightError(ValueError):
@@ -79,6 +83,10 @@ def read_tensors(
     wanted = {s.name: s for s in specs}
     missing = [n for n in wanted if n not in where]
     unexpected = [n for n in where if n not in wanted and n not in allow_unexpected]
+    ignored = [n for n in where if n not in wanted and n in allow_unexpected]
+    if ignored:
+        # the reference reads such a tensor's storage from the tensor it is tied to (llama.py:842-845)
+        log.warning("checkpoint in %s carries %s, which this model does not read: ignored", folder, ", ".join(sorted(ignored)))
     wrong_shape, wrong_type = [], []
     out: dict[str, torch.Tensor] = {}
     by_file: dict[Path, list[str]] = {}
