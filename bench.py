@@ -7,9 +7,13 @@ per sequence from the paged cache, sample, read the tokens back).  The default
 run has the layer sizes of Llama-3.2-1B with seeded random weights, 8 sequences
 and a context of 8192 tokens: each sequence's prompt is prefilled by the engine
 so that the timed steps end at the context length.  One JSON line is printed:
-``value`` is decoded tokens a second at batch 8; ``prefill`` is one 2,048-token
-prompt; ``roofline`` prices the decode step against the bytes it must read;
-``points`` holds decode at batch 1 and 64.
+``value`` is decoded tokens a second at batch 8 (from the mean step time, as the
+reference reports it, tokasaurus/benchmarks/bench_model.py:318-324); ``prefill`` is one
+2,048-token prompt (mean of 10); ``roofline`` prices the decode step against the bytes it
+must read; ``points`` holds decode at batch 1 and 64; ``timing`` gives mean, median and
+minimum of the timed iterations (the reference's timer, tokasaurus/utils.py:199-251);
+``measured`` holds two ceilings taken in the same process, a device copy of 1 GiB and one
+large bfloat16 product, and the fractions of them beside the fractions of the vendor's peaks.
 """
 
 from __future__ import annotations
@@ -74,21 +78,49 @@ SHAPES = {"1b": ("llama-3.2-1b-shape", LLAMA_1B), "3b": ("llama-3.2-3b-shape", L
 
 
 def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int, context: int, use_graphs: bool):
+    from tokasaurus_amd.engine.runner import ModelRunner
+
+    return ModelRunner.from_random(cfgd, 0, dtype, PAGE_SIZE, num_tokens // PAGE_SIZE, max_slots,
+                                   max_tokens_per_request=context, use_graphs=use_graphs,
+                                   graph_max_size=max(128, max_slots))
+
+
+def summary(ms: list[float]) -> dict:
+    """Mean, median and minimum of the timed iterations, in milliseconds."""
+    s = sorted(ms)
+    n = len(s)
+    median = s[n // 2] if n % 2 else 0.5 * (s[n // 2 - 1] + s[n // 2])
+    return {"mean": round(sum(s) / n, 4), "median": round(median, 4), "min": round(s[0], 4)}
+
+
+def measured_ceilings() -> dict:
+    """What this very device reaches on the two plainest workloads, for fractions that do not
+    lean on a data sheet: a device-to-device copy of 1 GiB (bytes read plus bytes written) and
+    one 8192 x 8192 x 8192 bfloat16 product of the library."""
     import torch
 
-    from tokasaurus_amd.engine.runner import DTYPES, ModelRunner, require_gpu
-    from tokasaurus_amd.models import architecture_of, build_model
-    from tokasaurus_amd.weights import draw_tensors
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end) / reps / 1e3
 
-    device = require_gpu()
-    arch = architecture_of(cfgd)
-    model = build_model(arch, arch.config_from_dict(cfgd))
-    tensors = draw_tensors(model.tensor_specs(), seed=0, device=device)
-    model.load(tensors, DTYPES[dtype], device)
-    del tensors
+    src = torch.empty((1 << 30,), dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    copy_s = timed(lambda: dst.copy_(src), 10)
+    del src, dst
+    n = 8192
+    a = torch.randn((n, n), dtype=torch.bfloat16, device="cuda")
+    b = torch.randn((n, n), dtype=torch.bfloat16, device="cuda")
+    gemm_s = timed(lambda: torch.mm(a, b.t()), 10)
+    del a, b
     torch.cuda.empty_cache()
-    return ModelRunner(model, PAGE_SIZE, num_tokens // PAGE_SIZE, max_slots, max_tokens_per_request=context,
-                       use_graphs=use_graphs, graph_max_size=max(128, max_slots))
+    return {"copy_gbs": round(2 * (1 << 30) / copy_s / 1e9, 1), "gemm_bf16_tflops": round(2.0 * n**3 / gemm_s / 1e12, 1)}
 
 
 def make_engine(runner, args, max_seqs: int):
@@ -151,30 +183,39 @@ def time_decode(runner, args, batch: int, ctx: int, steps: int, warmup: int) -> 
     assert len(engine.scheduler.decoding) == batch, (len(engine.scheduler.decoding), batch)
     for _ in range(warmup):
         engine.step()
+    # an event behind every step's launch: the device's own time from step to step
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
         engine.step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
+    per_step = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
     held = [rc.num_tokens for rc in runner.manager.requests.values()]
     assert len(held) == batch and max(held) <= ctx, (len(held), max(held), ctx)
     mean_ctx = sum(held) / len(held) - steps / 2  # mean over the timed steps
     for rid in list(engine.scheduler.decoding):
         engine.abort(rid)
     runner.manager.check()
-    say(f"batch {batch}: {dt * 1e3:.3f} ms a step, mean context {mean_ctx:.0f}")
-    return dt, mean_ctx
+    stats = summary(per_step)
+    say(f"batch {batch}: {dt * 1e3:.3f} ms a step by the host's clock around all {steps}, mean context {mean_ctx:.0f}; "
+        f"on the device mean {stats['mean']:.3f} median {stats['median']:.3f} min {stats['min']:.3f} ms")
+    return dt, mean_ctx, stats
 
 
-def time_prefill(runner, n: int, reps: int = 5) -> float:
+def time_prefill(runner, n: int, reps: int = 10) -> tuple[float, dict]:
+    """Seconds for one prompt of n tokens (the mean of `reps` runs after one untimed), and the
+    runs' mean, median and minimum in milliseconds."""
     import torch
 
     from tokasaurus_amd.engine.batch import StepEntry
 
     vocab = runner.model.spec.vocab_size
     toks = torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(1)).tolist()
-    best = float("inf")
+    times = []
     for i in range(reps + 1):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -183,8 +224,8 @@ def time_prefill(runner, n: int, reps: int = 5) -> float:
         dt = time.perf_counter() - t0
         runner.release("prefill")
         if i > 0:
-            best = min(best, dt)
-    return best
+            times.append(dt * 1e3)
+    return sum(times) / len(times) / 1e3, summary(times)
 
 
 def main() -> int:
@@ -206,14 +247,22 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
 
-    if args.prefill_only:
-        pdt = time_prefill(runner, PREFILL_TOKENS)
-        say(f"prefill of {PREFILL_TOKENS} tokens: {pdt * 1e3:.2f} ms")
+    def prefill_record(ceilings: dict | None) -> tuple[dict, dict]:
+        pdt, pstats = time_prefill(runner, PREFILL_TOKENS)
+        say(f"prefill of {PREFILL_TOKENS} tokens: mean {pstats['mean']:.2f} median {pstats['median']:.2f} min {pstats['min']:.2f} ms")
         flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], PREFILL_TOKENS)
-        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pdt, 1), "tokens": PREFILL_TOKENS, "ms": round(pdt * 1e3, 3),
-                                      "frac": round(flops / pdt / 1e12 / PEAK_TFLOPS[key], 4)}}))
+        rec = {"value": round(PREFILL_TOKENS / pdt, 1), "tokens": PREFILL_TOKENS, "ms": round(pdt * 1e3, 3),
+               "frac": round(flops / pdt / 1e12 / PEAK_TFLOPS[key], 4), "tflops": round(flops / pdt / 1e12, 1)}
+        if ceilings and key == "bf16":
+            rec["frac_of_measured"] = round(flops / pdt / 1e12 / ceilings["gemm_bf16_tflops"], 4)
+        return rec, pstats
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_record(None)[0]}))
         return 0
-    dt, mean_ctx = time_decode(runner, args, args.batch, args.context, args.steps, args.warmup)
+    ceilings = measured_ceilings()
+    say(f"measured ceilings: copy {ceilings['copy_gbs']} GB/s, bfloat16 product {ceilings['gemm_bf16_tflops']} TFLOP/s")
+    dt, mean_ctx, dstats = time_decode(runner, args, args.batch, args.context, args.steps, args.warmup)
     value = args.batch / dt
     nbytes = decode_bytes(runner.model, cfgd, args.batch, mean_ctx, elem)
     achieved = nbytes / dt / 1e9
@@ -258,23 +307,20 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "frac_of_measured": round(achieved / ceilings["copy_gbs"], 4),
         },
+        "measured": ceilings,
+        "timing": {"decode_ms": dstats},
     }
     if not args.no_prefill:
-        pdt = time_prefill(runner, PREFILL_TOKENS)
-        say(f"prefill of {PREFILL_TOKENS} tokens: {pdt * 1e3:.2f} ms")
-        flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], PREFILL_TOKENS)
-        out["prefill"] = {
-            "value": round(PREFILL_TOKENS / pdt, 1),
-            "tokens": PREFILL_TOKENS,
-            "ms": round(pdt * 1e3, 3),
-            "frac": round(flops / pdt / 1e12 / PEAK_TFLOPS[key], 4),
-        }
+        out["prefill"], out["timing"]["prefill_ms"] = prefill_record(ceilings)
     pts = {}
     for b in points:
         steps = max(8, min(args.steps, 32)) if b >= 32 else args.steps
-        pdt_b, _ = time_decode(runner, args, b, args.context, steps, args.warmup)
+        pdt_b, ctx_b, stats_b = time_decode(runner, args, b, args.context, steps, args.warmup)
         pts[f"decode_b{b}"] = round(b / pdt_b, 1)
+        out["timing"][f"decode_b{b}_ms"] = stats_b
+        out["timing"][f"decode_b{b}_hbm_frac"] = round(decode_bytes(runner.model, cfgd, b, ctx_b, elem) / pdt_b / 1e9 / HBM_PEAK_GBS, 4)
     out["points"] = pts
     print(json.dumps(out))
     return 0

@@ -38,3 +38,22 @@ def plain_generate(folder, prompt, max_tokens, temperature=0.0, engine_seed=0, r
         if tok in eos:
             break
     return out, lps
+
+
+def check_token_follows_plain(logits, tok: int, temperature: float, u: float, slack: float = 0.0) -> None:
+    """A token the bfloat16 engine chose, judged against the plain 32-bit logits of the same
+    history: rounding may flip a near tie but no more.  Greedy: the token's plain logit is within
+    0.08 (+ slack) of the best.  Sampled with the uniform number u: u lies within 0.05 (+ slack)
+    of the token's interval of cumulative plain probability (rounding moves the intervals' edges
+    by a few hundredths at most; a wrong distribution moves them anywhere)."""
+    import torch
+
+    if temperature == 0:
+        gap = float(logits.max() - logits[tok])
+        assert gap < 0.08 + slack, f"token {tok} is {gap:.3f} below the plain best {int(logits.argmax())}"
+        return
+    p = torch.softmax(logits.double() / temperature, -1)
+    hi = float(p[: tok + 1].sum())
+    lo = hi - float(p[tok])
+    tol = 0.05 + slack
+    assert lo - tol <= u <= hi + tol, f"token {tok} covers [{lo:.4f}, {hi:.4f}) of the plain distribution, u = {u:.4f}"

@@ -129,3 +129,47 @@ def compare_with_bfloat16_measure(got, plain: dict[str, torch.Tensor], plain16: 
                                  f"the plain model in bfloat16 (largest error {float(err.abs().max()):.3e})")
         worst = max(worst, ratio)
     return worst
+
+
+# --------------------------------------------------------------------------
+# faults put in on purpose: what the comparisons above must find
+# --------------------------------------------------------------------------
+
+
+def swap_pages(runner, rid_a: str, block_a: int, rid_b: str, block_b: int, group: int = 0) -> None:
+    """Exchange one page between the block tables of two live requests: every read stays
+    inside pages that the two own, but request a now sees a page of b's keys and values in
+    place of its own (and the other way round)."""
+    m = runner.manager
+    ra, rb = m.requests[rid_a], m.requests[rid_b]
+    pa, pb = ra.tables[group][block_a], rb.tables[group][block_b]
+    assert pa >= 0 and pb >= 0 and pa != pb
+    ra.tables[group][block_a], rb.tables[group][block_b] = pb, pa
+    if m.slot_tables is not None:
+        m.slot_tables[group][ra.slot, block_a] = pb
+        m.slot_tables[group][rb.slot, block_b] = pa
+
+
+def shift_position(runner, rid: str) -> None:
+    """The request's next token is taken to stand one position further than it does: it is
+    rotated for the wrong place and its key lands one slot too far, leaving a slot of zeros."""
+    rc = runner.manager.requests[rid]
+    runner.manager.reserve(rid, rc.num_tokens + 2)
+    rc.num_tokens += 1
+
+
+def faulty_tail(runner, reqs: dict[str, list[int]], victim: str, tail: int, fault) -> dict[tuple[str, int], torch.Tensor]:
+    """Every request's tokens but the victim's last ``tail`` go in honestly and unobserved; then
+    ``fault(runner)`` is applied and the victim's last tokens are decoded one by one.  Returns
+    their logits keyed as the plain rows are, (request, position the token truly has)."""
+    for rid, toks in reqs.items():
+        n = len(toks) - tail if rid == victim else len(toks)
+        runner.step([StepEntry(rid, toks[:n], [])])
+    fault(runner)
+    toks = reqs[victim]
+    got = {}
+    for pos in range(len(toks) - tail, len(toks)):
+        got[(victim, pos)] = runner.step([StepEntry(victim, [toks[pos]], [0])]).float().cpu()[0]
+    for rid in reqs:
+        runner.release(rid)
+    return got

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import plain_llama
-from gpu_common import plain_generate
+from gpu_common import check_token_follows_plain, plain_generate
 from tiny_models import CONFIG_A, PAGE_A, PAGE_B, TINY, make_folder, random_tokens
 from tokasaurus_amd import EngineConfig, SamplingParams
 from tokasaurus_amd.engine.engine import Engine
@@ -125,12 +125,12 @@ def test_bfloat16_generation_follows_the_plain_one(folders, name):
         # bfloat16 rounding of the best logit (a near tie may fall the other way)
         ids = list(prompt)
         for tok in c.tokens:
-            logits = plain_llama.forward_logits(pcfg, w, ids)[-1]
-            assert float(logits.max() - logits[tok]) < 0.08, (tok, int(logits.argmax()))
+            check_token_follows_plain(plain_llama.forward_logits(pcfg, w, ids)[-1], tok, 0.0, 0.0)
             ids.append(tok)
 
 
-def recorded_against_eager(folder, page, cfg, live, lengths, max_tokens, budget=None, padded=False):
+def recorded_against_eager(folder, page, cfg, live, lengths, max_tokens, budget=None, padded=False, graph_max_size=128,
+                           results_out=None):
     """The same requests through an engine with recorded decode steps and one without; returns
     the sizes that were recorded.  Requests end at different lengths, so the batch shrinks
     through the recorded sizes, each replayed several times with eager steps (prompt portions
@@ -145,6 +145,7 @@ def recorded_against_eager(folder, page, cfg, live, lengths, max_tokens, budget=
     for graphs in (True, False):
         engine = Engine(EngineConfig(
             model=str(folder), dtype="bfloat16", page_size=page, use_hipgraphs=graphs or padded, max_seqs_per_forward=live,
+            hipgraph_max_size=graph_max_size,
             max_tokens_per_forward=budget or max(32, live + 16), kv_cache_num_tokens=16384, allocator_sanity_checks=True))
         if padded and not graphs:
             engine.runner.capture_graphs = False
@@ -160,6 +161,8 @@ def recorded_against_eager(folder, page, cfg, live, lengths, max_tokens, budget=
     for (ta, la), (tb, lb) in zip(*results):
         assert ta == tb
         assert torch.allclose(torch.tensor(la), torch.tensor(lb), atol=1e-5)
+    if results_out is not None:
+        results_out.extend(zip(prompts, results[0]))
     return sizes
 
 
@@ -176,6 +179,44 @@ def test_recorded_and_eager_decode_steps_agree(folders, live, count):
     assert max(sizes) >= min(live, count) - 15
     if live == 128:
         assert {48, 64, 80, 96, 112, 128} <= sizes
+
+
+def test_decode_steps_of_more_rows_than_any_recorded_size(folders):
+    """160 live requests with recorded sizes up to 128: decode-only steps of 129 to 160 rows
+    are launched kernel by kernel, and as requests end the batch shrinks into the recorded
+    sizes.  The completions equal those of an engine that records nothing, and the chosen
+    tokens follow the plain model."""
+    cfg, page = TINY["C"]
+    count = 170
+    lengths = [4 + (7 * i) % 19 for i in range(count)]
+    out: list = []
+    seen_rows: list[int] = []
+    from tokasaurus_amd.engine import runner as runner_module
+
+    orig = runner_module.ModelRunner._recorded_for
+
+    def watching(self, planned):
+        step = orig(self, planned)
+        if step is None and planned and all(e.q_len == 1 for e in planned):
+            seen_rows.append(len(planned))
+        return step
+
+    runner_module.ModelRunner._recorded_for = watching
+    try:
+        sizes = recorded_against_eager(folders["C"], page, cfg, 160, lengths, lambda i: 5 + (5 * i) % 23, budget=2048,
+                                       graph_max_size=128, results_out=out)
+    finally:
+        runner_module.ModelRunner._recorded_for = orig
+    assert max(sizes) == 128
+    assert any(129 <= n <= 160 for n in seen_rows), "no decode-only step had more rows than the largest recorded size"
+    pcfg, w = plain_llama.load_folder(folders["C"])
+    for i in list(range(6)) + [count - 3, count - 2, count - 1]:
+        prompt, (tokens, _) = out[i]
+        ids = list(prompt)
+        for k, tok in enumerate(tokens[:6]):  # sampled at temperature 0.7 with the request's seed 3 + i
+            logits = plain_llama.forward_logits(pcfg, w, ids)[-1]
+            check_token_follows_plain(logits, tok, 0.7, uniform_for(0, 3 + i, k))
+            ids.append(tok)
 
 
 def test_finishing_on_an_end_token_and_on_length(folders, tmp_path):

@@ -8,7 +8,7 @@ import torch
 
 import plain_llama
 from gpu_common import TOL
-from replay_helpers import compare, mixed_trace, run_steps
+from replay_helpers import compare, faulty_tail, mixed_trace, run_steps, shift_position, swap_pages
 from tiny_models import make_folder, random_tokens
 from tokasaurus_amd.engine.runner import ModelRunner
 
@@ -69,6 +69,22 @@ def errors(got, plain, other=None):
     return (sq / n) ** 0.5, worst
 
 
+def check_against_plain_bfloat16(got, plain, plain16, largest_too=True):
+    """Six million logits through 2048-wide sums: the largest of so many rounding errors lies
+    beyond what the tiny models' bound allows for a few thousand.  The measure here is the plain
+    model computing in bfloat16 like the reference: the engine, which rounds in fewer places,
+    must not be further from the 32-bit logits than that, over all rows and row for row
+    (``largest_too``: also in the largest single error, a statistic for many rows only)."""
+    rms, worst = errors(got, plain)
+    rms16, worst16 = errors(got, plain, plain16)
+    print(f"engine: rms error {rms:.3e}, largest {worst:.3e}; plain bfloat16: rms error {rms16:.3e}, largest {worst16:.3e}")
+    assert rms <= rms16 and (worst <= worst16 or not largest_too), "further from the plain logits than the plain model in bfloat16"
+    for key, row in got.items():
+        r, _ = errors({key: row}, plain)
+        r16, _ = errors({key: row}, plain, plain16)
+        assert r <= 1.25 * r16, f"row {key}: {r:.3e} from the plain logits, the plain model in bfloat16 {r16:.3e}"
+
+
 def long_steps(tokens):
     head = LONG - 32
     steps = [{"entries": [("long", tokens[:head], LONG_WANT)]}]
@@ -89,23 +105,29 @@ def test_long_request_and_mixed_batches(model, dtype):
     assert max(len(s["entries"]) for s in steps) >= 3
     got.update(run_steps(runner, steps))
     assert len(got) == len(LONG_WANT) + 32 + sum(MIXED)
-    rms, worst = errors(got, plain)
-    print(f"{dtype}: rms error {rms:.3e}, largest {worst:.3e} against the plain 32-bit logits")
     if dtype == "float32":
         compare(got, plain, **TOL[dtype])
     else:
-        # Six million logits through 2048-wide sums: the largest of so many rounding errors
-        # lies beyond what the tiny models' bound allows for a few thousand.  The measure here is
-        # the plain model computing in bfloat16 like the reference: the engine, which rounds in
-        # fewer places, must not be further from the 32-bit logits than that, row for row.
-        rms16, worst16 = errors(got, plain, plain16)
-        print(f"plain bfloat16: rms error {rms16:.3e}, largest {worst16:.3e}")
-        assert rms <= rms16 and worst <= worst16
-        for key, row in got.items():
-            r, _ = errors({key: row}, plain)
-            r16, _ = errors({key: row}, plain, plain16)
-            assert r <= 1.25 * r16, (key, r, r16)
+        check_against_plain_bfloat16(got, plain, plain16)
     assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
+
+
+@pytest.mark.parametrize("fault", ["none", "page", "position"])
+def test_the_bfloat16_measure_finds_a_wrong_page_and_a_wrong_position(model, fault):
+    """One page of 16 keys among 600 taken from another request, or a decoded token one
+    position off: the measure that the bfloat16 run above passes must fail.  All reads stay
+    inside pages the two requests own; without a fault the same steps pass."""
+    folder, requests, plain, plain16 = model
+    reqs = {"long": requests["long"], "m0": requests["m0"]}
+    runner = ModelRunner.from_folder(folder, "bfloat16", page_size=PAGE, num_pages=(640 + 128) // PAGE, max_slots=4)
+    faults = {"none": lambda r: None, "page": lambda r: swap_pages(r, "long", 7, "m0", 2),
+              "position": lambda r: shift_position(r, "long")}
+    got = faulty_tail(runner, reqs, "long", 8, faults[fault])
+    if fault == "none":
+        check_against_plain_bfloat16(got, plain, plain16, largest_too=False)
+    else:
+        with pytest.raises(AssertionError, match="plain"):
+            check_against_plain_bfloat16(got, plain, plain16, largest_too=False)
 
 
 def test_recorded_steps_with_library_products_agree_with_eager_ones(model):

@@ -115,6 +115,50 @@ def test_llama3_scaling_bands():
     assert torch.allclose(lin, base / 4.0)
 
 
+@pytest.mark.parametrize("d, theta, factor, low, high, orig", [
+    (32, 500000.0, 8.0, 1.0, 4.0, 64),      # tiny configuration B
+    (64, 500000.0, 32.0, 1.0, 4.0, 8192),   # the 1B model's scaling
+    (128, 500000.0, 8.0, 1.0, 4.0, 8192),   # the 8B model's
+    (48, 10000.0, 4.0, 2.0, 8.0, 128),      # other factors: low_freq_factor is not 1
+])
+def test_llama3_blend_is_linear_in_frequency(d, theta, factor, low, high, orig):
+    """The middle band by the definition itself, element by element in Python floats:
+    s = (orig / wavelength - low) / (high - low) is linear in the FREQUENCY (not in the
+    wavelength) and the result is (1 - s) * f / factor + s * f.  A blend linear in the
+    wavelength, a blend of the angles' periods, or the two outer bands exchanged all fail this.
+    The reference delegates the generator to an installed package, which this build neither
+    reads nor imports: beyond this definition the parity of the blend is unpinned.  The
+    engine's own generator (a separate implementation) must give the same numbers."""
+    from tokasaurus_amd.parts.position import inverse_frequencies
+
+    sc = dict(rope_type="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high,
+              original_max_position_embeddings=orig)
+    want, bands = [], set()
+    for j in range(d // 2):
+        f = theta ** (-2.0 * j / d)
+        wavelength = 2.0 * math.pi / f
+        if wavelength < orig / high:
+            want.append(f)
+            bands.add("short")
+        elif wavelength > orig / low:
+            want.append(f / factor)
+            bands.add("long")
+        else:
+            s = (orig / wavelength - low) / (high - low)
+            assert 0.0 <= s <= 1.0
+            want.append((1.0 - s) * f / factor + s * f)
+            bands.add("middle")
+    assert bands == {"short", "long", "middle"}
+    want = torch.tensor(want, dtype=torch.float64)
+    for got in (pl.rope_inverse_frequencies(d, theta, sc), inverse_frequencies(d, theta, sc)):
+        assert got.dtype == torch.float32
+        assert torch.allclose(got.double(), want, rtol=2e-6, atol=0)
+    # at the band's two edges the blend meets the outer bands: s = 0 where the wavelength is
+    # orig / low and s = 1 where it is orig / high
+    for edge, s_want in ((orig / low, 0.0), (orig / high, 1.0)):
+        assert abs((orig / edge - low) / (high - low) - s_want) < 1e-12
+
+
 # ---- attention -------------------------------------------------------------
 
 

@@ -10,12 +10,13 @@ import torch
 
 import plain_llama
 import toy_parts
-from gpu_common import TOL, plain_generate
+from gpu_common import TOL, check_token_follows_plain, plain_generate
 from replay_helpers import compare, compare_with_bfloat16_measure, mixed_trace, plain_rows, run_steps
 from tiny_models import make_folder, random_tokens
 from tokasaurus_amd import EngineConfig, SamplingParams
 from tokasaurus_amd.engine.engine import Engine
 from tokasaurus_amd.engine.runner import ModelRunner
+from tokasaurus_amd.sampling import uniform_for
 
 pytestmark = pytest.mark.gpu
 
@@ -75,11 +76,15 @@ def test_a_random_configuration_in_mixed_batches(tmp_path, seed):
         assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("seed", [2, 8, 13, 21, 22, 23])
-def test_generation_under_random_options(tmp_path, seed):
+def test_generation_under_random_options(tmp_path, seed, dtype):
     """A random configuration under random engine options (page and cache size, budgets,
     portions, optimistic admission, paced prompts, a step ahead or not, recorded steps or not)
-    and random sampling options, in 32-bit: every completion is the plain one's."""
+    and random sampling options.  In 32-bit every completion is the plain one's.  In bfloat16
+    (the matrix-core kernels and recorded steps under bumping, pacing and a step ahead) every
+    chosen token follows the plain model given the engine's own history, and its
+    log-probability is the plain one's within what the plain model loses in bfloat16."""
     rng = random.Random(seed)
     cfg = random_config(rng)
     cfg["num_hidden_layers"] = min(cfg["num_hidden_layers"], 2)
@@ -91,7 +96,7 @@ def test_generation_under_random_options(tmp_path, seed):
                              seed=rng.randint(0, 999), topk_logprobs=rng.choice([None, 2])) for _ in range(n)]
     need = max(len(p) + sp.max_tokens for p, sp in zip(prompts, params))
     tokens = -(-rng.randint(need, 4 * need) // 64) * 64
-    options = dict(model=str(folder), dtype="float32", page_size=page, kv_cache_num_tokens=tokens,
+    options = dict(model=str(folder), dtype=dtype, page_size=page, kv_cache_num_tokens=tokens,
                    max_seqs_per_forward=rng.choice([2, 4, 8]), max_tokens_per_forward=rng.choice([16, 48, 128]),
                    max_prefill_chunk=rng.choice([None, 3, 16]), bump_city_population_me=rng.random() < 0.4,
                    greedy_prefill=rng.random() < 0.6, prefill_round_up_multiple=rng.choice([1, 4, 16]),
@@ -100,11 +105,28 @@ def test_generation_under_random_options(tmp_path, seed):
     print(f"seed {seed}: {cfg}\n{options}")
     engine = Engine(EngineConfig(**options))
     done = engine.generate(prompts, params)
+    if dtype == "bfloat16":
+        pcfg, w = plain_llama.load_folder(folder)
+        cfg16, w16 = plain_llama.load_folder(folder, torch.bfloat16)
     for c, prompt, sp in zip(done, prompts, params):
-        want, want_lp = plain_generate(folder, prompt, sp.max_tokens, temperature=sp.temperature, engine_seed=seed,
-                                       request_seed=sp.seed)
-        assert c.tokens == want
-        assert torch.allclose(torch.tensor(c.logprobs), torch.tensor(want_lp), atol=2e-4)
+        if dtype == "float32":
+            want, want_lp = plain_generate(folder, prompt, sp.max_tokens, temperature=sp.temperature, engine_seed=seed,
+                                           request_seed=sp.seed)
+            assert c.tokens == want
+            assert torch.allclose(torch.tensor(c.logprobs), torch.tensor(want_lp), atol=2e-4)
+        else:
+            assert len(c.tokens) == sp.max_tokens
+            ids = list(prompt)
+            for k, (tok, lp) in enumerate(zip(c.tokens, c.logprobs)):
+                logits = plain_llama.forward_logits(pcfg, w, ids)[-1]
+                # what rounding costs at this width: the plain model in bfloat16 on the same history
+                lost = float((plain_llama.forward_logits(cfg16, w16, ids)[-1] - logits).abs().max())
+                u = uniform_for(seed, sp.seed, k) if sp.temperature > 0 else 0.0
+                check_token_follows_plain(logits, tok, sp.temperature, u, slack=2 * lost)
+                t = sp.temperature if sp.temperature > 0 else 1.0
+                plain_lp = float(torch.log_softmax(logits / t, -1)[tok])
+                assert abs(lp - plain_lp) <= (0.06 + 2 * lost) / min(t, 1.0), (k, tok, lp, plain_lp)
+                ids.append(tok)
         assert (c.topk_ids is None) == (sp.topk_logprobs is None)
         if c.topk_ids is not None:
             assert [len(t) for t in c.topk_ids] == [2] * len(c.tokens)

@@ -12,7 +12,8 @@ import torch
 
 import plain_llama
 from gpu_common import TOL
-from replay_helpers import compare, mixed_trace, plain_rows, portions, run_steps, tail_one_by_one, whole
+from replay_helpers import (compare, faulty_tail, mixed_trace, plain_rows, portions, run_steps, shift_position, swap_pages,
+                            tail_one_by_one, whole)
 from tiny_models import TINY, random_tokens
 from tokasaurus_amd.cache import NoSpaceException
 from tokasaurus_amd.engine.batch import StepEntry
@@ -167,6 +168,32 @@ def test_no_space_leaves_the_cache_usable(folders):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("fault", ["none", "page", "position"])
+def test_the_bounds_find_a_wrong_page_and_a_wrong_position(folders, name, dtype, fault):
+    """The comparison with the plain logits must fail when one page of a request's block
+    table names another request's page, and when a decoded token stands one position off:
+    otherwise the bound (of bfloat16 above all) would let such faults of the cache through.
+    Every access stays inside pages the two requests own.  Without a fault the same steps pass."""
+    cfg, page = TINY[name]
+    reqs = {"v": random_tokens(120, cfg["vocab_size"], 31), "w": random_tokens(70, cfg["vocab_size"], 32)}
+    ref = plain_rows(folders[name], reqs)
+    runner = runner_for(folders, name, dtype)
+    faults = {
+        "none": lambda r: None,
+        # one page of 120 tokens' worth: 4 keys of 112 in configuration A, 16 in C
+        "page": lambda r: swap_pages(r, "v", 40 // page, "w", 1),
+        "position": lambda r: shift_position(r, "v"),
+    }
+    got = faulty_tail(runner, reqs, "v", 8, faults[fault])
+    if fault == "none":
+        compare(got, ref, **TOL[dtype])
+    else:
+        with pytest.raises(AssertionError, match="plain"):
+            compare(got, ref, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_trace_run_program(folders, tmp_path, dtype):
     """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done' lines out."""
     cfg, page = TINY["B"]
@@ -192,6 +219,10 @@ def test_trace_run_program(folders, tmp_path, dtype):
     for step, rows in expect.items():
         arr = np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, V)
         assert arr.shape[0] == len(rows)
+        # beside the logits, the rows' names: request id and position of every row
+        named = json.loads((out / f"{step}.json").read_text())
+        assert named["step"] == step and named["vocab"] == V
+        assert [tuple(r) for r in named["rows"]] == rows
         got = {key: torch.from_numpy(arr[i].copy()) for i, key in enumerate(rows)}
         compare(got, ref, **TOL[dtype])
 

@@ -452,3 +452,15 @@ def test_fresh_slots_are_reported_once():
         run_step(s)
     reused = cache.take_fresh_slots()
     assert len(reused) == 1 and reused[0] in (0, 1)  # c took a slot that a or b gave back
+
+
+def test_state_counts_of_the_stats_line():
+    s, cache = make(num_pages=16, page_size=4, max_tokens_per_forward=8, max_seqs=2)
+    s.submit(req("a", 6, 7))   # life 12 tokens: 3 pages, 2 for the prompt
+    s.submit(req("b", 3, 2))   # life 4 tokens: 1 page
+    s.submit(req("c", 3, 2))   # waits: two requests may run
+    run_step(s)                # a: 6 prompt tokens, b: 2 of its 3
+    c = s.state_counts()
+    assert (c["num_running_seqs"], c["num_decoding_seqs"], c["num_prefilling_seqs"], c["num_queued_seqs"]) == (2, 1, 1, 1)
+    assert c["kv_cache_frac_allocated"] == 3 / 16 and c["kv_cache_frac_reserved"] == 1 / 16
+    assert c["kv_cache_frac_total"] == 4 / 16 and c["mean_running_seq_len"] == (6 + 2) / 2

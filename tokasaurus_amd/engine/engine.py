@@ -44,7 +44,9 @@ class Completion:
 
 @dataclass
 class Stats:
-    """The counters of the reference's stats line (tokasaurus/manager/monitoring.py:179-232)."""
+    """The counters of the reference's stats line (tokasaurus/manager/monitoring.py:179-232);
+    ``extra`` holds the measurements of the current state (monitoring.py:297-325), which the
+    engine refreshes whenever it reports."""
 
     steps: int = 0
     prefill_tokens: int = 0
@@ -67,6 +69,7 @@ class Stats:
             "total_tok_per_s": total / s,
             "tok_per_forward": total / max(self.steps, 1),
             "forwards_per_s": self.steps / s,
+            **self.extra,
         }
 
 
@@ -211,6 +214,11 @@ class Engine:
         self.stats.seconds += time.perf_counter() - t0
         return done
 
+    def report(self) -> dict:
+        """The stats line: throughput so far and the state of cache and queues right now."""
+        self.stats.extra = self.scheduler.state_counts()
+        return self.stats.as_dict()
+
     def run_until_done(self) -> list[Completion]:
         """Step until nothing is left; every ``stats_report_seconds`` a line of counters goes to
         the log (the reference's stats line, tokasaurus/manager/monitoring.py:179-232)."""
@@ -220,7 +228,7 @@ class Engine:
             done.extend(self.step())
             if self.config.stats_report_seconds > 0 and time.perf_counter() - last >= self.config.stats_report_seconds:
                 last = time.perf_counter()
-                log.info("stats %s", {k: (round(v, 1) if isinstance(v, float) else v) for k, v in self.stats.as_dict().items()})
+                log.info("stats %s", {k: (round(v, 3) if isinstance(v, float) else v) for k, v in self.report().items()})
         return done
 
     def generate(self, prompts: list[list[int]], params: SamplingParams | list[SamplingParams] | None = None) -> list[Completion]:

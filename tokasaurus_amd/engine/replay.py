@@ -5,7 +5,9 @@ own: it drives the ``ModelRunner`` that generation uses.
 Input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
 For a step in which something is wanted, ``<out>/<step>.f32`` holds the logits at
-the wanted places as little-endian float32 [wanted, vocab].  After every step
+the wanted places as little-endian float32 [wanted, vocab], and ``<out>/<step>.json``
+names the rows: ``{"step": s, "vocab": V, "rows": [[request id, position], ...]}``, the
+position being the token's place in its request counted from 0.  After every step
 the line ``done <step>`` is printed and flushed.
 """
 
@@ -57,10 +59,16 @@ def run(args: argparse.Namespace, lines=None, out=None) -> int:
         entries = [StepEntry(str(e["id"]), [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])])
                    for e in rec.get("entries", [])]
         if entries:
+            # a row's position: the tokens its request held before this step plus the wanted place
+            held = {e.request_id: (runner.manager.requests[e.request_id].num_tokens
+                                   if e.request_id in runner.manager.requests else 0) for e in entries}
             logits = runner.step(entries)
             if logits.shape[0] > 0:
                 arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                 np.ascontiguousarray(arr).tofile(out_dir / f"{rec['step']}.f32")
+                rows = [[e.request_id, held[e.request_id] + w] for e in entries for w in e.want]
+                (out_dir / f"{rec['step']}.json").write_text(
+                    json.dumps({"step": rec["step"], "vocab": int(arr.shape[1]), "rows": rows}) + "\n")
         for rid in rec.get("end", []):
             # a request that never held anything (or was ended before) has nothing to give back
             if str(rid) in runner.manager.requests:

@@ -340,6 +340,34 @@ class ModelRunner:
         model.load(tensors, DTYPES[dtype], device)
         return cls(model, page_size, num_pages, max_slots, **options)
 
+    @classmethod
+    def from_random(
+        cls,
+        config: dict,
+        seed: int,
+        dtype: str,
+        page_size: int,
+        num_pages: int,
+        max_slots: int,
+        **options,
+    ) -> "ModelRunner":
+        """A runner on seeded random weights drawn on the device, for models too large to be
+        worth a folder (benchmarks): ``config`` is what config.json would hold; the values are
+        those of ``weights.draw_tensors`` with the device's generator."""
+        from tokasaurus_amd.models.registry import architecture_of
+        from tokasaurus_amd.weights.random_init import draw_tensors
+
+        device = require_gpu()
+        if dtype not in DTYPES:
+            raise ValueError(f"dtype {dtype!r}: this engine runs {sorted(DTYPES)}")
+        arch = architecture_of(config)
+        model = build_model(arch, arch.config_from_dict(config))
+        tensors = draw_tensors(model.tensor_specs(), seed=seed, device=device)
+        model.load(tensors, DTYPES[dtype], device)
+        del tensors
+        torch.cuda.empty_cache()
+        return cls(model, page_size, num_pages, max_slots, **options)
+
     # ---- requests
     def admit(self, request_id: str) -> None:
         self.manager.admit(request_id)

@@ -158,6 +158,28 @@ class Scheduler:
         """Pages a running request may still claim (manager/types.py:94-104)."""
         return max(0, self.cache.blocks_for(req.max_cache_tokens()) - self._held_blocks(req))
 
+    def state_counts(self) -> dict:
+        """The measurements of the current state that the reference's stats line carries beside
+        its throughput (tokasaurus/manager/monitoring.py:297-325): the fraction of the cache's
+        pages that requests hold, the fraction that running requests may still claim, and how
+        many requests run, decode, prefill and wait."""
+        running = self.running()
+        total = min((pool.num_pages for pool in self.cache.pools), default=0)
+        held = total - min(self.cache.num_free_pages(), default=0)
+        claimed = sum(self._outstanding(r) for r in running)
+        lens = [r.cache_tokens() for r in running]
+        frac = (lambda n: n / total) if total else (lambda n: 0.0)
+        return {
+            "kv_cache_frac_allocated": frac(held),
+            "kv_cache_frac_reserved": frac(claimed),
+            "kv_cache_frac_total": frac(held + claimed),
+            "num_running_seqs": len(running),
+            "num_decoding_seqs": len(self.decoding),
+            "num_prefilling_seqs": len(self.prefilling),
+            "num_queued_seqs": len(self.queued),
+            "mean_running_seq_len": sum(lens) / len(lens) if lens else 0.0,
+        }
+
     # ---- one scheduling round
     def schedule(self) -> Decision:
         self._make_room_for_decoding()

@@ -99,7 +99,9 @@ class Linear:
                                             prenorm=prenorm, norm_eps=eps)
             # library matrix product (hipBLASLt), 32-bit accumulation
             if residual is not None:
-                return torch.addmm(residual, x, w.t())  # the residual is added in the product's epilogue
+                # the product is rounded to the storage type before the residual is added, as in the
+                # few-row kernel and in the pass that adds and norms (and as the reference's separate add)
+                return ops.add(torch.mm(x, w.t()), residual.contiguous())
             if out_f32:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
             prod = torch.mm(x, w.t())
