@@ -1,0 +1,458 @@
+// Device code of the matrix-core attention, shared by the attention kernel and by kernels
+// that run attention as one of their phases.  See attention_mfma.hip for the method.
+#pragma once
+
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+// Accesses that are coherent across the chip's dies (each has an L2 of its own): relaxed
+// atomics of agent scope, which the compiler turns into loads that go around, and stores that
+// write through, the caches.  Data that one workgroup of a running kernel writes and another
+// reads moves through these; no cache-wide write-back or invalidation is needed then.
+__device__ __forceinline__ uint64_t shared_load64(const void* p) {
+  return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void shared_store64(void* p, uint64_t v) {
+  __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void shared_store16(void* p, uint16_t v) {
+  __hip_atomic_store((uint16_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <bool SHARED>
+__device__ __forceinline__ bf16x8_t load_bf16x8(const bf16_t* p) {
+  if constexpr (SHARED) {
+    union { uint64_t u[2]; bf16x8_t v; } x;
+    x.u[0] = shared_load64(p);
+    x.u[1] = shared_load64(p + 4);
+    return x.v;
+  } else {
+    return *(const bf16x8_t*)p;
+  }
+}
+template <bool SHARED>
+__device__ __forceinline__ void store_f32x4(float* p, f32x4_t v) {
+  if constexpr (SHARED) {
+    union { uint64_t u[2]; f32x4_t v; } x;
+    x.v = v;
+    shared_store64(p, x.u[0]);
+    shared_store64(p + 2, x.u[1]);
+  } else {
+    *(f32x4_t*)p = v;
+  }
+}
+template <bool SHARED>
+__device__ __forceinline__ void store_f32x2(float* p, float a, float b) {
+  if constexpr (SHARED) {
+    union { uint64_t u; float f[2]; } x;
+    x.f[0] = a;
+    x.f[1] = b;
+    shared_store64(p, x.u);
+  } else {
+    p[0] = a;
+    p[1] = b;
+  }
+}
+
+struct AttnArgs {
+  const bf16_t* q;
+  int q_stride;
+  bf16_t* out;
+  int out_stride;
+  const bf16_t* kcache;
+  const bf16_t* vcache;
+  const int* block_table;
+  int table_stride;
+  const int* q_start;   // [requests + 1]
+  const int* kv_len;    // [requests]
+  const int* tile_req;  // [tiles]
+  const int* tile_row0; // [tiles] first row of the wavefront's first row tile
+  const int* tile_row1; // [tiles] first row of its second row tile, -1 for none; null: the 16 rows after the first
+  int n_tiles;
+  int nq, nkv, group, P, p_shift, window;
+  float scale_log2;  // scale * log2(e) > 0
+  int split;         // keys per split, a multiple of 32
+  int max_splits;    // splits a tile may have (size of the scratch)
+  float* part_o;     // [tiles][nkv][max_splits][16 * RT][D]
+  float* part_ml;    // [tiles][nkv][max_splits][16 * RT][2]
+};
+
+// What a (wavefront's) tile covers.  Per row tile: rows row0 .. row0 + 15 (row0 < 0: none),
+// keys [lo, hi] that some row sees and [full_lo, full_hi] that every row sees.
+struct TileRange {
+  int req, qs, qlen, kvl, n_rows, lo, hi, s_first, s_last;
+  int row0[2], rt_lo[2], rt_hi[2], full_lo[2], full_hi[2];
+};
+
+__device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int row_tiles) {
+  TileRange t;
+  // a null tile list stands for one token a request, each a tile of its own
+  t.req = a.tile_req ? a.tile_req[tile] : tile;
+  t.qs = a.tile_req ? a.q_start[t.req] : t.req;
+  t.qlen = a.tile_req ? a.q_start[t.req + 1] - t.qs : 1;
+  t.kvl = a.kv_len[t.req];
+  t.n_rows = t.qlen * a.group;
+  t.row0[0] = a.tile_req ? a.tile_row0[tile] : 0;
+  t.row0[1] = -1;
+  if (row_tiles == 2) {
+    t.row0[1] = a.tile_row1 ? a.tile_row1[tile] : t.row0[0] + 16;
+    if (t.row0[1] >= t.n_rows) t.row0[1] = -1;
+  }
+  t.lo = 0x7fffffff;
+  t.hi = -1;
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    t.rt_lo[rt] = t.full_lo[rt] = 0x7fffffff;
+    t.rt_hi[rt] = t.full_hi[rt] = -1;
+    if (t.row0[rt] < 0) continue;
+    const int first_tok = t.row0[rt] / a.group;
+    const int last_tok = min(t.row0[rt] + 15, t.n_rows - 1) / a.group;
+    const int pos_first = t.kvl - t.qlen + first_tok, pos_last = t.kvl - t.qlen + last_tok;
+    t.rt_hi[rt] = pos_last;
+    t.rt_lo[rt] = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+    t.full_hi[rt] = pos_first;
+    t.full_lo[rt] = a.window > 0 ? max(0, pos_last - a.window + 1) : 0;
+    t.lo = min(t.lo, t.rt_lo[rt]);
+    t.hi = max(t.hi, t.rt_hi[rt]);
+  }
+  t.s_first = t.lo / a.split;
+  t.s_last = t.hi / a.split;
+  return t;
+}
+
+// first <= x <= last as one unsigned comparison (an empty range, last < first, holds nothing)
+struct Range {
+  int first;
+  unsigned span;
+  __device__ __forceinline__ bool holds(int x) const { return (unsigned)(x - first) <= span; }
+};
+__device__ __forceinline__ Range range_of(int first, int last) {
+  return last >= first ? Range{first, (unsigned)(last - first)} : Range{0x7fffffff, 0u};
+}
+
+// The maximum over the four lanes (r, 0..3) that share a row: lanes 16 and 32 apart,
+// with the gfx950 swaps of 16-lane rows and of wavefront halves.
+__device__ __forceinline__ float max_over_quarters(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const unsigned v = __float_as_uint(y);
+  const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+// The loads of one step of 32 keys.  Keys: lane (r, q) reads 8 values of key
+// kb + 16 blk + r for every 32-wide step over the head size.  Values: lane (r, q)
+// reads, for d = 16 dt + r, the 4 keys kb + 16 blk + 4q .. + 3.  Every address lies
+// in a page of the tile's key range [lo, hi], so a load past the end reads valid
+// memory (whose contents the masks keep out of the result).
+template <int DT>
+struct StepRegs {
+  bf16x8_t kv[2][(DT + 1) / 2];
+  union { bf16x4_t half[2]; uint32_t u[4]; bf16x8_t whole; } vv[DT];  // the two 16-key blocks side by side
+};
+
+// BIG: pages of 16 keys or more, so the 16 keys of a block lie in one page, which a
+// scalar load looks up; the lane's part of the address is the same in every step.
+// The pages of the two 16-key blocks of the step at `kb` (BIG only): looked up a step before
+// the loads that need them are issued, so that no load waits for a table entry.
+struct StepPages {
+  int page[2];
+};
+
+__device__ __forceinline__ StepPages step_pages(const AttnArgs& a, const int* table, int kb, int lo, int hi) {
+  const int sh = a.p_shift;
+  StepPages p;
+  p.page[0] = table[min(max(kb >> sh, lo >> sh), hi >> sh)];
+  p.page[1] = table[min(max((kb + 16) >> sh, lo >> sh), hi >> sh)];
+  return p;
+}
+
+template <int DT, bool BIG>
+__device__ __forceinline__ void load_step(StepRegs<DT>& s, const AttnArgs& a, const int* table, const StepPages& pages,
+                                          int kvh, int kb, int lo, int hi, int r, int q) {
+  constexpr int D = DT * 16;
+  constexpr int KS = (DT + 1) / 2;
+  const int P = a.P, sh = a.p_shift;
+  // the lane's own part of a key and of a value address inside any page of this kv head
+  const unsigned lane_k = (unsigned)(kvh * P * D + r * 8);
+  const unsigned lane_v = (unsigned)(kvh * P * D + (q * D + r) * 4);
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const bf16_t* kp;
+    const bf16_t* vp;
+    if constexpr (BIG) {
+      const int key0 = kb + blk * 16;
+      // one 32 x 32 -> 64-bit product a page: the kv head's offset is in the lane's part already
+      const size_t base = (size_t)(unsigned)pages.page[blk] * (unsigned)(a.nkv * P * D);
+      const int in_page = key0 & (P - 1);
+      kp = a.kcache + base + (unsigned)(in_page * 8) + lane_k;
+      vp = a.vcache + base + (unsigned)((in_page >> 2) * (D * 4)) + lane_v;
+    } else {
+      const int kk = min(max(kb + blk * 16 + r, lo), hi);
+      const int page = table[kk >> sh];
+      kp = a.kcache + ((size_t)page * a.nkv + kvh) * ((size_t)P * D) + (size_t)(kk & (P - 1)) * 8;
+      int kc = kb + blk * 16 + q * 4;
+      if (kc > hi) kc = hi & ~3;
+      if (kc + 3 < lo) kc = lo & ~3;
+      const int vpage = table[kc >> sh];
+      vp = a.vcache + ((size_t)vpage * a.nkv + kvh) * ((size_t)P * D) + (size_t)((kc & (P - 1)) >> 2) * (D * 4) + r * 4;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + q * 8;  // piece d0 / 8 of the key
+      if (d0 < D) {
+        s.kv[blk][ks] = *(const bf16x8_t*)(kp + (size_t)(d0 >> 3) * P * 8);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s.kv[blk][ks][e] = (__bf16)0.f;
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) s.vv[dt].half[blk] = *(const bf16x4_t*)(vp + dt * 64);
+  }
+}
+
+// Wavefronts a workgroup may have: the fewer, the more registers each has for loads in flight.
+__host__ __device__ constexpr int max_waves(int dt, int rt) { return rt == 2 ? 4 : (dt <= 4 ? 16 : 8); }
+
+// One (tile, kv head, split) item of the attention: the body of the kernel, for the NW
+// wavefronts of a workgroup together (all of them must call it: it synchronises them when
+// NW > 1).  wg_part is LDS of NW * 16 * RT * (D + 4) floats (unused when NW is 1).
+// SHARED: the item runs inside a kernel whose workgroups hand data to each other (a persistent
+// kernel): queries are read and results written with accesses that are coherent across the
+// chip, and the result always goes to the partial buffers, also when the tile has one split.
+// PF steps of loads are in flight: a lone wavefront on a long tile waits on memory otherwise.
+template <int DT, int RT, bool BIG, bool SHARED>
+__device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile, const int kvh, const int split_index,
+                                               float* wg_part, const int NW) {
+  constexpr int D = DT * 16;
+  constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head size
+  constexpr int PF = RT == 1 ? 2 : 3;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  const TileRange t = tile_range(a, tile, RT);
+  const int s = t.s_first + split_index;
+  if (s > t.s_last) return;
+  const int nsp = t.s_last - t.s_first + 1;
+  // this wavefront's part of the split: `sub` keys, a multiple of 32
+  const int sub = a.split / NW;
+  const int k_begin = max((t.lo >> 5) << 5, s * a.split + wave * sub);
+  const int k_end = min(t.hi + 1, s * a.split + (wave + 1) * sub);
+  const int* table = a.block_table + (size_t)t.req * a.table_stride;
+
+  // the steps (by their first key) in which a row tile has a row that sees a key, in which all
+  // of its rows see all 32 keys, and in which all 32 keys lie in the tile's range
+  Range active[RT], unmasked[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    active[rt] = range_of(t.rt_lo[rt] - 31, t.rt_hi[rt]);
+    unmasked[rt] = range_of(t.full_lo[rt], t.full_hi[rt] - 31);
+  }
+  const Range inside = range_of(t.lo, t.hi - 31);
+
+  // this lane's row in each of the RT tiles
+  int pos_r[RT], lo_r[RT], flat_r[RT];
+  bf16x8_t qv[RT][KS];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int flat = t.row0[rt] >= 0 ? t.row0[rt] + r : t.n_rows;
+    const bool valid = flat < t.n_rows;
+    flat_r[rt] = valid ? flat : -1;
+    const int fl = valid ? flat : t.n_rows - 1;
+    const int tok = fl / a.group, g = fl - tok * a.group;
+    const int pos = t.kvl - t.qlen + tok;
+    pos_r[rt] = valid ? pos : -1;
+    lo_r[rt] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    const bf16_t* qp = a.q + (size_t)(t.qs + tok) * a.q_stride + (size_t)(kvh * a.group + g) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + q * 8;
+      if (d0 < D) {
+        qv[rt][ks] = load_bf16x8<SHARED>(qp + d0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[rt][ks][e] = (__bf16)0.f;
+      }
+    }
+  }
+
+  float m_run[RT], l_run[RT];  // running maximum of the row's products and sum of this lane's keys
+  f32x4_t acc[RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    m_run[rt] = -INFINITY;
+    l_run[rt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  auto compute_step = [&](StepRegs<DT>& cur, const int kb) {
+    if (!inside.holds(kb)) {
+      // values of keys outside the tile's range may be anything (a freed page): make them
+      // zero by masking their 16 bits
+      uint32_t keep[4];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int key = kb + blk * 16 + q * 4 + 2 * h;
+          const uint32_t lo16 = (key >= t.lo && key <= t.hi) ? 0x0000ffffu : 0u;
+          const uint32_t hi16 = (key + 1 >= t.lo && key + 1 <= t.hi) ? 0xffff0000u : 0u;
+          keep[blk * 2 + h] = lo16 | hi16;
+        }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) cur.vv[dt].u[i] &= keep[i];
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if (!active[rt].holds(kb)) continue;  // none of the tile's rows sees these keys
+      f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        st[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[0][ks], qv[rt][ks], st[0], 0, 0, 0);
+        st[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.kv[1][ks], qv[rt][ks], st[1], 0, 0, 0);
+      }
+      // scores stay as the products are (scale_log2 > 0 keeps their order); the scale goes
+      // into the exponent's multiply-add
+      float sc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc[e] = st[e >> 2][e & 3];
+      if (!unmasked[rt].holds(kb)) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int key = kb + (e >> 2) * 16 + q * 4 + (e & 3);
+          if (!(key >= lo_r[rt] && key <= pos_r[rt])) sc[e] = -INFINITY;
+        }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      mx = max_over_quarters(mx);
+      const float m_new = fmaxf(m_run[rt], mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float mc = m_use * a.scale_log2;
+      if (__any(m_new > m_run[rt])) {
+        // some row's maximum moved: weigh what was summed so far
+        const float alpha = __builtin_amdgcn_exp2f(fmaf(m_run[rt], a.scale_log2, -mc));  // 0 while nothing was seen
+        l_run[rt] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[rt][dt] *= alpha;
+        m_run[rt] = m_new;
+      }
+      float psum = 0.f;
+      bf16x8_t pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(fmaf(sc[e], a.scale_log2, -mc));
+        psum += p;
+        pb[e] = (__bf16)p;
+      }
+      l_run[rt] += psum;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        acc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vv[dt].whole, pb, acc[rt][dt], 0, 0, 0);
+    }
+  };
+
+  StepRegs<DT> ring[PF];
+  // With two row tiles (prompts: many steps a wavefront) the pages of a step are looked up when
+  // the loads of the step before are issued; with one (decode: few steps) right before its own.
+  constexpr bool AHEAD = BIG && RT == 2;
+  StepPages pages = {};
+  if (AHEAD && k_begin < k_end) pages = step_pages(a, table, k_begin, t.lo, t.hi);
+  auto issue = [&](StepRegs<DT>& regs, int k) {
+    if (BIG && !AHEAD) pages = step_pages(a, table, k, t.lo, t.hi);
+    load_step<DT, BIG>(regs, a, table, pages, kvh, k, t.lo, t.hi, r, q);
+    if (AHEAD && k + 32 < k_end) pages = step_pages(a, table, k + 32, t.lo, t.hi);
+  };
+#pragma unroll
+  for (int i = 0; i < PF; ++i)
+    if (k_begin + 32 * i < k_end) issue(ring[i], k_begin + 32 * i);
+  for (int kb = k_begin; kb < k_end; kb += 32 * PF) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int k = kb + 32 * i;
+      if (k < k_end) {
+        compute_step(ring[i], k);
+        if (k + 32 * PF < k_end) issue(ring[i], k + 32 * PF);
+      }
+    }
+  }
+
+  // acc[rt][dt][j] of lane (r, q) is O^T[d = 16 dt + 4q + j][row r]
+  const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float l = l_run[rt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    l_run[rt] = l;
+    m_run[rt] *= a.scale_log2;  // from here on in units of log 2, as the merges take it
+  }
+  if (NW > 1) {
+    // every wavefront leaves (max, sum, weighted values) of its rows; wavefront 0 adds them in order
+    constexpr int ROW = D + 4;  // max, sum, two unused, then the values (16-byte aligned)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float* row = wg_part + ((size_t)wave * 16 * RT + rt * 16 + r) * ROW;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *(f32x4_t*)(row + 4 + dt * 16 + q * 4) = acc[rt][dt];
+      if (q == 0) {
+        row[0] = m_run[rt];
+        row[1] = l_run[rt];
+      }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float m = -INFINITY;
+      for (int w = 0; w < NW; ++w) m = fmaxf(m, wg_part[((size_t)w * 16 * RT + rt * 16 + r) * ROW]);
+      float l = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int w = 0; w < NW; ++w) {
+        const float* row = wg_part + ((size_t)w * 16 * RT + rt * 16 + r) * ROW;
+        const float mw = row[0];
+        const float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
+        l += f * row[1];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[rt][dt] += f * *(const f32x4_t*)(row + 4 + dt * 16 + q * 4);
+      }
+      m_run[rt] = m;
+      l_run[rt] = l;
+    }
+  }
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const float l = l_run[rt];
+    const int flat = flat_r[rt];
+    if (flat < 0) continue;
+    if (nsp == 1 && !SHARED) {
+      const int tok = flat / a.group, g = flat - tok * a.group;
+      bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;
+      const float inv = 1.0f / l;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        union { bf16_t h[4]; uint2 u; } pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pk.h[j] = __float2bfloat16(acc[rt][dt][j] * inv);
+        *(uint2*)(op + dt * 16 + q * 4) = pk.u;
+      }
+    } else {
+      const size_t item = item0 + (s - t.s_first);
+      float* po = a.part_o + (item * (16 * RT) + rt * 16 + r) * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) store_f32x4<SHARED>(po + dt * 16 + q * 4, acc[rt][dt]);
+      if (q == 0) {
+        float* pm = a.part_ml + (item * (16 * RT) + rt * 16 + r) * 2;
+        store_f32x2<SHARED>(pm, m_run[rt], l);
+      }
+    }
+  }
+}

@@ -75,6 +75,14 @@ __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return __float2bfl
 template <typename T>
 __device__ __forceinline__ float round_to(float v) { return to_f32<T>(from_f32<T>(v)); }
 
+// silu(gate) * up as the engine's storage type sees it: both operands and the activation
+// rounded to bfloat16, the product left in 32-bit for the caller to round.
+__device__ __forceinline__ float silu_mul_bf16(float g, float u) {
+  const float gr = round_to<bf16_t>(g), ur = round_to<bf16_t>(u);
+  const float s = round_to<bf16_t>(gr / (1.0f + expf(-gr)));
+  return s * ur;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = TK_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TK_WAVE);

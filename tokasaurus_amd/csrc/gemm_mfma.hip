@@ -73,12 +73,6 @@ struct GemmArgs {
   int TH;       // weight rows of a tile that are used (16, or 8 to make twice the workgroups of a narrow output)
 };
 
-__device__ __forceinline__ float silu_mul_bf16(float g, float u) {
-  const float gr = round_to<bf16_t>(g), ur = round_to<bf16_t>(u);
-  const float s = round_to<bf16_t>(gr / (1.0f + expf(-gr)));
-  return s * ur;
-}
-
 template <int EPI>
 __device__ __forceinline__ void store4(const GemmArgs& a, f32x4_t v, f32x4_t up, float scale, int token, int n) {
   if (token >= a.M) return;

@@ -27,7 +27,7 @@ CSRC = Path(__file__).resolve().parent.parent / "csrc"
 IN_TREE_DIR = Path(__file__).resolve().parent / "_build"
 GROUPS = {
     "core": ["errors.hip", "elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sample.hip"],
-    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip"],
+    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip", "decode_layers.hip"],
 }
 
 ARCH = "gfx950"
@@ -48,7 +48,8 @@ HIPCC_FLAGS = [
 
 # The attention kernel rescales its accumulators between matrix products: they stay in
 # ordinary vector registers instead of moving to and from the accumulation registers.
-SOURCE_FLAGS = {"attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+SOURCE_FLAGS = {"attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+                "decode_layers.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
 
 class BuildError(RuntimeError):
