@@ -49,6 +49,9 @@ class EngineConfig:
     use_hipgraphs: bool = True
     hipgraph_max_size: int = 128
     hipgraph_step: int = 16
+    # experimental: decode steps of up to 16 requests run the blocks of the model in ONE kernel
+    # (one workgroup a compute unit, barriers across the grid) instead of six kernels a block
+    fuse_decode_layers: bool = False
 
     # --- steps launched before their tokens are back (tokasaurus/common_types.py:89; the
     # reference queues up to 8 between two processes, this loop keeps at most one ahead:

@@ -223,8 +223,9 @@ __host__ __device__ constexpr int max_waves(int dt, int rt) { return rt == 2 ? 4
 // wavefronts of a workgroup together (all of them must call it: it synchronises them when
 // NW > 1).  wg_part is LDS of NW * 16 * RT * (D + 4) floats (unused when NW is 1).
 // SHARED: the item runs inside a kernel whose workgroups hand data to each other (a persistent
-// kernel): queries are read and results written with accesses that are coherent across the
-// chip, and the result always goes to the partial buffers, also when the tile has one split.
+// kernel): results are written with stores that write through the caches, and always to the
+// partial buffers, also when the tile has one split (queries are read as ever: such a kernel
+// keeps them in a buffer that is written once in a launch).
 // PF steps of loads are in flight: a lone wavefront on a long tile waits on memory otherwise.
 template <int DT, int RT, bool BIG, bool SHARED>
 __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile, const int kvh, const int split_index,
@@ -273,7 +274,7 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
     for (int ks = 0; ks < KS; ++ks) {
       const int d0 = ks * 32 + q * 8;
       if (d0 < D) {
-        qv[rt][ks] = load_bf16x8<SHARED>(qp + d0);
+        qv[rt][ks] = *(const bf16x8_t*)(qp + d0);
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[rt][ks][e] = (__bf16)0.f;

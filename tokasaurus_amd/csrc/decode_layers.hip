@@ -20,9 +20,13 @@
 //
 // Data between workgroups (the residual stream, q, the attention's partial results, the
 // gate|up result, the new key and value in the pages) is written with stores that write
-// through the caches and read with loads that go around them (agent-scope relaxed atomics),
-// because each of the chip's eight dies has an L2 of its own; the grid barrier then needs no
-// cache-wide write-back or invalidation, only a wait for the workgroup's own stores.
+// through the caches (agent-scope relaxed atomics), because each of the chip's eight dies has
+// an L2 of its own; the grid barrier then needs no cache-wide write-back, only a wait for the
+// workgroup's own stores.  It is read with ordinary cached loads, which is sound because every
+// block has scratch buffers of its own: within a launch a buffer is written once and read only
+// behind the barrier that follows, so no cache can hold a line of it from before the write (and
+// a launch starts with clean caches).  Reading around the caches instead would send every
+// workgroup's read of the same few KB to the one or two memory channels that hold them.
 //
 // The grid barrier: workgroups arrive at a counter of their group of 16, the last of a group
 // at the top counter, the last there raises every group's flag, which the group's workgroups
@@ -41,6 +45,7 @@
 #define DL_FAN 16             // workgroups per first-level counter of the barrier
 #define DL_MAX_GROUPS 4096    // workgroups a launch may have
 #define DL_MAX_TABLES 4       // block tables (cache groups) a run of blocks may use
+#define DL_MARKS_PER_LAYER 24  // timing marks a block may leave
 
 // words of the sync buffer (uint32), 16 apart so that each sits in a cache line of its own
 #define DL_SYNC_GROUP(g) (16 * (g))
@@ -75,12 +80,13 @@ struct DecodeArgs {
   const int* kv_len;     // [M] keys of each request after this step's append (position + 1)
   const int* tables[DL_MAX_TABLES];  // block tables [M, stride]
   int table_stride[DL_MAX_TABLES];
-  bf16_t* x;   // [M, H] the residual stream: in, and out after the last block
-  bf16_t* xb;  // [M, H] scratch: the stream between mixer and feed-forward
-  bf16_t* q;   // [M, nq d] scratch
-  bf16_t* h;   // [M, I] scratch
-  float* part_o;   // [M][nkv][max_splits][16][d] partial attention results
-  float* part_ml;  // [M][nkv][max_splits][16][2]
+  // scratch, one buffer a block each (a buffer is written once in a launch):
+  bf16_t* xs;   // [n_layers + 1][M, H] the residual stream: xs[0] in, xs[l + 1] out of block l
+  bf16_t* xbs;  // [n_layers][M, H] the stream between mixer and feed-forward
+  bf16_t* qs;   // [n_layers][M, nq d]
+  bf16_t* hs;   // [n_layers][M, I]
+  float* part_o;   // [n_layers][M][nkv][max_splits][16][d] partial attention results
+  float* part_ml;  // [n_layers][M][nkv][max_splits][16][2]
   int split, max_splits;
   float scale;
   // for the norm that follows the run (null: none): x * w rounded once, and per row one
@@ -93,9 +99,9 @@ struct DecodeArgs {
   uint32_t* status;  // set to non-zero when a wait gave up
   uint32_t spin_cap;
   uint32_t expect_groups;  // workgroups the barrier waits for (the grid's size; tests pass one more)
-  // diagnostics (null: none): workgroup `timing_group` writes the constant-rate clock (100 MHz)
-  // at the start and, per block, after each of the 5 phases and each of the 5 barriers:
-  // 1 + 10 * n_layers words
+  // diagnostics (null: none): workgroup `timing_group` writes pairs (mark id, constant-rate clock
+  // of 100 MHz) at the start and at up to DL_MARKS_PER_LAYER places of every block:
+  // 2 * (1 + DL_MARKS_PER_LAYER * n_layers) words
   unsigned long long* timing;
   int timing_group;
 };
@@ -186,10 +192,25 @@ __device__ __forceinline__ bf16x8_t dl_zero8() {
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 
 // LDS of a product phase: [ssq: DL_WAVES x 16 floats][sums: (PAIRED ? 2 : 1) x tiles x DL_WAVES x 64 f32x4]
+// (the output product keeps the merged attention, its operand, behind the sums)
 #define DL_SSQ_FLOATS (DL_WAVES * 16)
+#define DL_RED_FLOATS (DL_MAX_TILES * DL_WAVES * 64 * 4)
 
 struct PhaseShape {
   int u0, u1, nt, th;  // this workgroup's units [u0, u1), in nt tiles of th units
+};
+
+// Diagnostics: one thread of one workgroup leaves (id, clock) pairs.
+struct Marks {
+  unsigned long long* out;  // null: off
+  int at, limit;
+  __device__ __forceinline__ void operator()(int id) {
+    if (out != nullptr && at < limit) {
+      out[2 * at] = (unsigned long long)id;
+      out[2 * at + 1] = wall_clock64();
+      ++at;
+    }
+  }
 };
 
 __device__ __forceinline__ PhaseShape phase_shape(int units) {
@@ -203,94 +224,165 @@ __device__ __forceinline__ PhaseShape phase_shape(int units) {
   return p;
 }
 
-// C[token][unit] = sum_k A[token][k] W[row(unit)][k] for this workgroup's units.
+// One wavefront's share of a product phase.  C[token][unit] = sum_k A[token][k] W[row(unit)][k]
+// for the workgroup's units; the wavefront takes the steps ks0 .. ks0 + n_steps - 1 of K (32
+// values a step) of every tile: n_slots = nt * n_steps (tile, step) slots, in chunks of 8.
 //   PAIRED: a unit is two rows, row(unit) and row(unit) + pair_off; `half` > 0 maps unit u to
 //   row (u / half) * 2 half + u % half (the first of a rotation's pair), else row = unit.
-//   load_a(step, first_pass) gives lane (token r, quarter q) its 8 values A[r][32 step + 8 q ..];
+#define DL_CHUNK 8
+struct Share {
+  const bf16_t* W;
+  const bf16_t* zeros;  // 16 bytes of zeros in device memory: what a lane without a weight row reads
+  PhaseShape p;
+  int K, half, pair_off, ks0, n_steps, n_slots, n_chunks;
+};
+
+__device__ __forceinline__ Share make_share(const bf16_t* W, const bf16_t* zeros, int K, int units, int half, int pair_off,
+                                            int wave) {
+  Share s;
+  s.W = W; s.zeros = zeros; s.K = K; s.half = half; s.pair_off = pair_off;
+  s.p = phase_shape(units);
+  const int K32 = (K + 31) >> 5;
+  s.ks0 = K32 * wave / DL_WAVES;
+  s.n_steps = K32 * (wave + 1) / DL_WAVES - s.ks0;
+  s.n_slots = s.p.nt * s.n_steps;
+  s.n_chunks = (s.n_slots + DL_CHUNK - 1) / DL_CHUNK;
+  return s;
+}
+
+template <bool PAIRED>
+struct WChunk {
+  bf16x8_t a[DL_CHUNK];
+  bf16x8_t b[PAIRED ? DL_CHUNK : 1];
+};
+
+__device__ __forceinline__ bf16x8_t keep_if(bool ok, bf16x8_t v) {
+  union { bf16x8_t v; uint32_t u[4]; } x;
+  x.v = v;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) x.u[e] = ok ? x.u[e] : 0u;
+  return x.v;
+}
+
+// The weights of chunk `chunk`: every lane loads, from an address that always exists (a slot or
+// a lane without a weight row reads 16 bytes of zeros), so that the loads of a chunk are
+// straight-line code whose arrival the hardware's counter tells apart, and nothing has to
+// touch a loaded value before the matrix core does.
+template <bool PAIRED>
+__device__ __forceinline__ void load_weights(WChunk<PAIRED>& c, const Share& s, int chunk, int r, int q) {
+  const int n_steps = max(s.n_steps, 1);
+  int tile = chunk * DL_CHUNK / n_steps, si = chunk * DL_CHUNK - tile * n_steps;
+#pragma unroll
+  for (int j = 0; j < DL_CHUNK; ++j) {
+    const int unit = s.p.u0 + tile * s.p.th + r, k0 = (s.ks0 + si) * 32 + q * 8;
+    const bool ok = tile < s.p.nt && r < s.p.th && unit < s.p.u1 && k0 < s.K;
+    const int uu = ok ? unit : 0;
+    const int row = s.half > 0 ? (uu / s.half) * (2 * s.half) + uu % s.half : uu;
+    const bf16_t* ptr = s.W + (size_t)row * s.K + k0;
+    c.a[j] = *(const bf16x8_t*)(ok ? ptr : s.zeros);
+    if (PAIRED) c.b[j] = *(const bf16x8_t*)(ok ? ptr + (size_t)s.pair_off * s.K : s.zeros);
+    if (++si == n_steps) { si = 0; ++tile; }
+  }
+}
+
+template <bool PAIRED>
+__device__ __forceinline__ void zero_weights(WChunk<PAIRED>& c) {
+#pragma unroll
+  for (int j = 0; j < DL_CHUNK; ++j) {
+    c.a[j] = dl_zero8();
+    if (PAIRED) c.b[j] = dl_zero8();
+  }
+}
+
+// The weights of a share, NB chunks deep.  begin() asks for the first NB chunks and may be called
+// long before the product runs (before the barrier that the product's other operand waits for:
+// weights do not depend on it); the product asks for chunk c + NB when it has multiplied chunk c.
+template <bool PAIRED, int NB>
+struct WeightStream {
+  WChunk<PAIRED> buf[NB];
+  Share s;
+  __device__ __forceinline__ void begin(const bf16_t* W, const bf16_t* zeros, int K, int units, int half, int pair_off,
+                                        int wave, int r, int q) {
+    s = make_share(W, zeros, K, units, half, pair_off, wave);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      if (i < s.n_chunks) load_weights<PAIRED>(buf[i], s, i, r, q);
+      else zero_weights<PAIRED>(buf[i]);
+    }
+  }
+};
+
+// The product of a stream whose first chunks begin() has asked for.
+//   load_a(step, first_pass) gives lane (token r, quarter q) its 8 values A[r][32 step + 8 q ..]
+//   for ANY step (it reads an address that exists and drops what lies past the end);
 //   first_pass is true in the workgroup's first tile (statistics of A are taken there, once).
+//   The operands of a chunk are asked for while the chunk before it is multiplied.
 //   before_sync(): called by every wavefront after its last product, before the workgroup's
-//   barrier (statistics go to LDS here).
+//   barrier (statistics go to LDS here; the next phase's weights are asked for here).
 //   epilogue(token, slot, unit0, limit, s0, s1): the sums of units unit0 .. unit0 + 3 (those
 //   below `limit` exist) for one token, s1 the paired rows'; slot = tile * 4 + quarter numbers
 //   the calls of one token.
-template <bool PAIRED, typename LoadA, typename BeforeSync, typename Epilogue>
-__device__ __forceinline__ void product_phase(const bf16_t* __restrict__ W, const int K, const int units, const int half,
-                                              const int pair_off, float* lds, LoadA load_a, BeforeSync before_sync,
-                                              Epilogue epilogue) {
-  const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, q = lane >> 4;
+template <bool PAIRED, int NB, typename LoadA, typename BeforeSync, typename Epilogue>
+__device__ __forceinline__ void product_run(WeightStream<PAIRED, NB>& ws, float* lds, Marks& mark, int mark_id, int r, int q,
+                                            LoadA load_a, BeforeSync before_sync, Epilogue epilogue) {
+  static_assert(NB == 1 || NB % 2 == 0, "the operand buffers alternate: an even number of weight buffers, or one");
+  const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const PhaseShape p = phase_shape(units);
-  const int K32 = (K + 31) >> 5;
-  const int ks0 = K32 * wave / DL_WAVES, ks1 = K32 * (wave + 1) / DL_WAVES;
-  const int n_steps = ks1 - ks0;
-  const int n_slots = p.nt * n_steps;
+  const Share s = ws.s;
+  const PhaseShape p = s.p;
+  const int n_steps = max(s.n_steps, 1);
   f32x4_t* red = (f32x4_t*)(lds + DL_SSQ_FLOATS);
   f32x4_t* red2 = red + p.nt * DL_WAVES * 64;
 
-  // the weight row of this lane in a tile
-  auto row_of = [&](int tile, bool& ok) -> const bf16_t* {
-    const int unit = p.u0 + tile * p.th + r;
-    ok = r < p.th && unit < p.u1;
-    const int uu = ok ? unit : p.u0;
-    const int row = half > 0 ? (uu / half) * (2 * half) + uu % half : uu;
-    return W + (size_t)row * K + q * 8;
+  bf16x8_t av[2][DL_CHUNK];
+  auto load_operands = [&](bf16x8_t (&dst)[DL_CHUNK], int chunk) {
+    int tile = chunk * DL_CHUNK / n_steps, si = chunk * DL_CHUNK - tile * n_steps;
+#pragma unroll
+    for (int j = 0; j < DL_CHUNK; ++j) {
+      dst[j] = load_a(s.ks0 + si, tile == 0);
+      if (++si == n_steps) { si = 0; ++tile; }
+    }
   };
-
-  bf16x8_t wa[DL_RING], wb[DL_RING], av[DL_RING];
-  int i_tile = 0, i_step = 0;
-  bool ok_i = false;
-  const bf16_t* p_i = p.nt > 0 ? row_of(0, ok_i) : W;
-  auto issue = [&](bf16x8_t& w0, bf16x8_t& w1, bf16x8_t& a0) {
-    if (i_tile < p.nt && n_steps > 0) {
-      const int step = ks0 + i_step;
-      const bool ok = ok_i && step * 32 + q * 8 < K;
-      if (ok) {
-        w0 = *(const bf16x8_t*)(p_i + (size_t)step * 32);
-        if (PAIRED) w1 = *(const bf16x8_t*)(p_i + (size_t)pair_off * K + (size_t)step * 32);
-      } else {
-        w0 = dl_zero8();
-        if (PAIRED) w1 = dl_zero8();
-      }
-      a0 = load_a(step, i_tile == 0);
-      if (++i_step == n_steps) {
-        i_step = 0;
-        ++i_tile;
-        if (i_tile < p.nt) p_i = row_of(i_tile, ok_i);
+  f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
+  int c_tile = 0, c_step = 0;
+  auto multiply = [&](const WChunk<PAIRED>& w, const bf16x8_t (&a)[DL_CHUNK], int chunk) {
+#pragma unroll
+    for (int j = 0; j < DL_CHUNK; ++j) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.a[j], a[j], acc0, 0, 0, 0);
+      if (PAIRED) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.b[PAIRED ? j : 0], a[j], acc1, 0, 0, 0);
+      if (chunk * DL_CHUNK + j < s.n_slots && ++c_step == s.n_steps) {
+        red[(c_tile * DL_WAVES + wave) * 64 + lane] = acc0;
+        if (PAIRED) red2[(c_tile * DL_WAVES + wave) * 64 + lane] = acc1;
+        acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        acc1 = acc0;
+        c_step = 0;
+        ++c_tile;
       }
     }
   };
-#pragma unroll
-  for (int j = 0; j < DL_RING; ++j) issue(wa[j], wb[j], av[j]);
 
-  f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
-  int c_tile = 0, c_step = 0;
-  for (int base = 0; base < n_slots; base += DL_RING) {
+  if (s.n_chunks > 0) load_operands(av[0], 0);
+  for (int c = 0; c < s.n_chunks; c += (NB == 1 ? 2 : NB)) {
 #pragma unroll
-    for (int j = 0; j < DL_RING; ++j) {
-      if (base + j < n_slots) {
-        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], av[j], acc0, 0, 0, 0);
-        if (PAIRED) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[j], av[j], acc1, 0, 0, 0);
-        if (++c_step == n_steps) {
-          red[(c_tile * DL_WAVES + wave) * 64 + lane] = acc0;
-          if (PAIRED) red2[(c_tile * DL_WAVES + wave) * 64 + lane] = acc1;
-          acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f};
-          acc1 = acc0;
-          c_step = 0;
-          ++c_tile;
-        }
-        issue(wa[j], wb[j], av[j]);
+    for (int i = 0; i < (NB == 1 ? 2 : NB); ++i) {
+      if (c + i < s.n_chunks) {
+        if (c + i + 1 < s.n_chunks) load_operands(av[(i + 1) & 1], c + i + 1);
+        multiply(ws.buf[i % NB], av[i & 1], c + i);
+        if (c + i + NB < s.n_chunks) load_weights<PAIRED>(ws.buf[i % NB], s, c + i + NB, r, q);
       }
     }
   }
-  if (n_steps == 0) {
+  if (s.n_steps == 0) {
     // a wavefront without a part of K still owes its (zero) sums
     for (int t = 0; t < p.nt; ++t) {
       red[(t * DL_WAVES + wave) * 64 + lane] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       if (PAIRED) red2[(t * DL_WAVES + wave) * 64 + lane] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
   }
+  mark(mark_id);  // products done
   before_sync();
   __syncthreads();
+  mark(mark_id + 1);  // sums of all wavefronts in LDS
   for (int u = tid; u < p.nt * 64; u += DL_THREADS) {
     const int l = u & 63, t = u >> 6;
     f32x4_t s0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, s1 = s0;
@@ -306,39 +398,43 @@ __device__ __forceinline__ void product_phase(const bf16_t* __restrict__ W, cons
 }
 
 // lane (token r, quarter q): 8 values of a [M, K] bfloat16 matrix written by other workgroups
-__device__ __forceinline__ bf16x8_t load_rows(const bf16_t* A, int lda, int M, int K, int step, int r, int q) {
+__device__ __forceinline__ bf16x8_t load_rows(const bf16_t* A, const bf16_t* zeros, int lda, int M, int K, int step, int r,
+                                              int q) {
   const int k0 = step * 32 + q * 8;
-  if (r >= M || k0 >= K) return dl_zero8();
-  return load_bf16x8<true>(A + (size_t)r * lda + k0);
+  const bool ok = r < M && k0 < K;
+  return *(const bf16x8_t*)(ok ? A + (size_t)r * lda + k0 : zeros);
 }
 
 // The operand of a product behind an RMSNorm: x * w rounded once (the rows are divided by their
 // rms after the product), and the sum of x^2 over what this lane saw.
-__device__ __forceinline__ bf16x8_t load_normed(const bf16_t* x, int H, int M, const void* w, int w_f32, int step, int r,
-                                                int q, bool first, float& ssq) {
+__device__ __forceinline__ bf16x8_t load_normed(const bf16_t* x, const bf16_t* zeros, int H, int M, const void* w, int w_f32,
+                                                int step, int r, int q, bool first, float& ssq) {
   const int k0 = step * 32 + q * 8;
-  if (r >= M || k0 >= H) return dl_zero8();
-  union { uint64_t u[2]; uint16_t h[8]; } xv;
-  xv.u[0] = shared_load64(x + (size_t)r * H + k0);
-  xv.u[1] = shared_load64(x + (size_t)r * H + k0 + 4);
+  const bool ok = r < M && k0 < H;
+  const int kk = ok ? k0 : 0;
+  union { uint4 u; uint16_t h[8]; } xv;
+  const bf16_t* xp = ok ? x + (size_t)r * H + k0 : zeros;
+  xv.u = *(const uint4*)xp;
   float wv[8];
   if (w_f32) {
-    const f32x4_t a = *(const f32x4_t*)((const float*)w + k0), b = *(const f32x4_t*)((const float*)w + k0 + 4);
+    const f32x4_t a = *(const f32x4_t*)((const float*)w + kk), b = *(const f32x4_t*)((const float*)w + kk + 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) { wv[e] = a[e]; wv[4 + e] = b[e]; }
   } else {
     union { uint4 u; uint16_t h[8]; } ww;
-    ww.u = *(const uint4*)((const bf16_t*)w + k0);
+    ww.u = *(const uint4*)((const bf16_t*)w + kk);
 #pragma unroll
     for (int e = 0; e < 8; ++e) wv[e] = bf16_bits_to_f32(ww.h[e]);
   }
   bf16x8_t out;
+  float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float xr = bf16_bits_to_f32(xv.h[e]);
-    if (first) ssq = fmaf(xr, xr, ssq);
+    ss = fmaf(xr, xr, ss);
     out[e] = (__bf16)(wv[e] * xr);
   }
+  if (first) ssq += ss;
   return out;
 }
 
@@ -376,9 +472,92 @@ __device__ __forceinline__ void store_row4(bf16_t* row, int n, int limit, const 
   }
 }
 
+// four values of a bfloat16 row that other workgroups wrote (those below `limit`; else 0)
+__device__ __forceinline__ void load_row4(const bf16_t* row, int n, int limit, float (&o)[4]) {
+  if (n + 3 < limit && (n & 3) == 0 && (((uintptr_t)row) & 7) == 0) {
+    union { uint64_t u; uint16_t h[4]; } pk;
+    pk.u = *(const uint64_t*)(row + n);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = bf16_bits_to_f32(pk.h[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[j] = 0.f;
+      if (n + j < limit) o[j] = __bfloat162float(row[n + j]);
+    }
+  }
+}
+
+// The attention's splits of every (token, head) merged, in split order, into the operand of
+// the output product, in LDS in the order the matrix core's lanes read it: the 8 values of
+// (step, lane = quarter * 16 + token) lie together.  All the workgroup's threads take part; the
+// partial results of up to DL_MAX_SPLITS splits are asked for at once.
+#define DL_MAX_SPLITS 16
+template <int D>
+__device__ __forceinline__ void merge_attention(const DecodeArgs& a, const float* part_o, const float* part_ml, int window,
+                                                bf16_t* stage) {
+  const int M = a.M, nq = a.nq, nkv = a.nkv, group = nq / nkv, K = nq * D;
+  const int K32 = (K + 31) >> 5;
+  // the columns past K of the last step must be zero (their weights are, and 0 * garbage may be NaN);
+  // rows of tokens past M stay as they are: they reach no output that is kept
+  for (int it = threadIdx.x; it < 16 * (K32 * 32 - K) / 4; it += DL_THREADS) {
+    const int token = it & 15, k = K + (it >> 4) * 4;
+    *(uint64_t*)(stage + ((size_t)((k >> 5) * 64 + ((k & 31) >> 3) * 16 + token) * 8 + (k & 7))) = 0;
+  }
+  const int chunks = K / 4;  // K is a multiple of 8
+  for (int it = threadIdx.x; it < M * chunks; it += DL_THREADS) {
+    const int token = it / chunks, k = (it - token * chunks) * 4;
+    union { uint64_t u; uint16_t h[4]; } pk;
+    const int head = k / D, c0 = k - head * D;
+    const int kvh = head / group, row = head - kvh * group;
+    const int kvl = a.kv_len[token];
+    const int lo = window > 0 ? max(0, kvl - window) : 0;
+    const int s_first = lo / a.split, nsp = (kvl - 1) / a.split - s_first + 1;
+    const size_t item0 = ((size_t)token * nkv + kvh) * a.max_splits;
+    const float* ml = part_ml + (item0 * 16 + row) * 2;
+    const float* po = part_o + (item0 * 16 + row) * D + c0;
+    union { uint64_t u; float f[2]; } mlv[DL_MAX_SPLITS], pa[DL_MAX_SPLITS], pb[DL_MAX_SPLITS];
+#pragma unroll
+    for (int sp = 0; sp < DL_MAX_SPLITS; ++sp) {
+      if (sp < nsp) {
+        mlv[sp].u = *(const uint64_t*)(ml + (size_t)sp * 32);
+        pa[sp].u = *(const uint64_t*)(po + (size_t)sp * 16 * D);
+        pb[sp].u = *(const uint64_t*)(po + (size_t)sp * 16 * D + 2);
+      }
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int sp = 0; sp < DL_MAX_SPLITS; ++sp)
+      if (sp < nsp) m = fmaxf(m, mlv[sp].f[0]);
+    float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sp = 0; sp < DL_MAX_SPLITS; ++sp) {
+      if (sp < nsp) {
+        const float w = mlv[sp].f[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mlv[sp].f[0] - m);
+        l += w * mlv[sp].f[1];
+        o[0] += w * pa[sp].f[0];
+        o[1] += w * pa[sp].f[1];
+        o[2] += w * pb[sp].f[0];
+        o[3] += w * pb[sp].f[1];
+      }
+    }
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pk.h[j] = bf16_bits(o[j] * inv);
+    const int step = k >> 5, qq = (k & 31) >> 3;
+    *(uint64_t*)(stage + ((size_t)(step * 64 + qq * 16 + token) * 8 + (k & 7))) = pk.u;
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------
+// chunks (of 8 slots) of weights a wavefront asks for ahead, per product
+#define DL_AHEAD_QKV 1
+#define DL_AHEAD_O 1
+#define DL_AHEAD_GU 2
+#define DL_AHEAD_DOWN 2
+
 template <int DT, bool BIG>
 __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a) {
   extern __shared__ __align__(16) float lds[];
@@ -388,32 +567,67 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
   const int M = a.M, H = a.H, I = a.I, nq = a.nq, nkv = a.nkv, P = a.P;
   const int half = D / 2, group = nq / nkv;
   GridSync gs = grid_sync_begin(a);
-  const bool timed = a.timing != nullptr && (int)blockIdx.x == a.timing_group && tid == 0;
-  if (timed) a.timing[0] = wall_clock64();
-  int mark_at = 1;
-  auto mark = [&]() {
-    if (timed) a.timing[mark_at] = wall_clock64();
-    ++mark_at;
-  };
+  const bf16_t* zeros = (const bf16_t*)(a.sync + 4);  // words 4 .. 7 of the sync buffer are never written
+  Marks mark;
+  mark.out = (a.timing != nullptr && (int)blockIdx.x == a.timing_group && tid == 0) ? a.timing : nullptr;
+  mark.at = 0;
+  mark.limit = 1 + DL_MARKS_PER_LAYER * a.n_layers;
+  mark(0);
+
+  WeightStream<true, DL_AHEAD_QKV> w_qkv;
+  WeightStream<false, DL_AHEAD_O> w_o;
+  WeightStream<true, DL_AHEAD_GU> w_gu;
+  WeightStream<false, DL_AHEAD_DOWN> w_down;
+  if (a.n_layers > 0) w_qkv.begin(a.layers[0].w_qkv, zeros, H, (nq + 2 * nkv) * half, half, half, wave, r, q);
 
   for (int li = 0; li < a.n_layers; ++li) {
     const DecodeLayer L = a.layers[li];
     const int* table = a.tables[L.table];
     const int table_stride = a.table_stride[L.table];
     const bool last_layer = li + 1 == a.n_layers;
+    // this block's scratch
+    const bf16_t* x_in = a.xs + (size_t)li * M * H;
+    bf16_t* x_out = a.xs + (size_t)(li + 1) * M * H;
+    bf16_t* xb = a.xbs + (size_t)li * M * H;
+    bf16_t* qbuf = a.qs + (size_t)li * M * nq * D;
+    bf16_t* hbuf = a.hs + (size_t)li * M * I;
+    const size_t part_items = (size_t)M * nkv * a.max_splits * 16;
+    float* part_o = a.part_o + (size_t)li * part_items * D;
+    float* part_ml = a.part_ml + (size_t)li * part_items * 2;
 
     // ---- 1. q | k | v of the normed stream, rotated; q to scratch, k and v to the pages
     {
+      // what the rotation of this thread's first four units reads, asked for ahead of the product
+      const PhaseShape shape = w_qkv.s.p;
+      int pre_pos = 0, pre_page = 0;
+      float pre_cs[4] = {1.f, 1.f, 1.f, 1.f}, pre_sn[4] = {0.f, 0.f, 0.f, 0.f};
+      if (tid < shape.nt * 64 && (tid & 15) < M) {
+        const int token = tid & 15;
+        pre_pos = a.positions[token];
+        pre_page = table[(size_t)token * table_stride + pre_pos / P];
+        const int unit0 = shape.u0 + (tid >> 6) * shape.th + ((tid & 63) >> 4) * 4;
+        const int limit = min(shape.u1, shape.u0 + ((tid >> 6) + 1) * shape.th);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int unit = unit0 + j;
+          if (unit < limit && unit / half < nq + nkv && L.cos_t != nullptr) {
+            pre_cs[j] = L.cos_t[(size_t)pre_pos * half + unit % half];
+            pre_sn[j] = L.sin_t[(size_t)pre_pos * half + unit % half];
+          }
+        }
+      }
       float ssq = 0.f;
-      product_phase<true>(
-          L.w_qkv, H, (nq + 2 * nkv) * half, half, half, lds,
-          [&](int step, bool first) { return load_normed(a.x, H, M, L.norm1, L.norm1_f32, step, r, q, first, ssq); },
+      product_run(
+          w_qkv, lds, mark, 10, r, q,
+          [&](int step, bool first) { return load_normed(x_in, zeros, H, M, L.norm1, L.norm1_f32, step, r, q, first, ssq); },
           [&]() { put_ssq(lds, ssq, wave, lane); },
-          [&](int token, int, int unit0, int limit, f32x4_t s0, f32x4_t s1) {
+          [&](int token, int slot, int unit0, int limit, f32x4_t s0, f32x4_t s1) {
             if (token >= M) return;
             const float rstd = rstd_of(lds, token, H, L.eps1);
-            const int pos = a.positions[token];
-            const int page = table[(size_t)token * table_stride + pos / P];
+            // this thread's first call is the one it asked ahead for: (tile, quarter, token) = its own thread number
+            const bool pre = (slot >> 2) * 64 + (slot & 3) * 16 + token == tid;
+            const int pos = pre ? pre_pos : a.positions[token];
+            const int page = pre ? pre_page : table[(size_t)token * table_stride + pos / P];
             const int off = pos % P;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -422,10 +636,13 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
               const int head = unit / half, c = unit - head * half;
               const float x1 = round_to<bf16_t>(s0[j] * rstd), x2 = round_to<bf16_t>(s1[j] * rstd);
               float o1 = x1, o2 = x2;
-              if (head < nq + nkv && L.cos_t != nullptr)
-                rotate_pair(x1, x2, L.cos_t[(size_t)pos * half + c], L.sin_t[(size_t)pos * half + c], o1, o2);
+              if (head < nq + nkv && L.cos_t != nullptr) {
+                const float cs = pre ? pre_cs[j] : L.cos_t[(size_t)pos * half + c];
+                const float sn = pre ? pre_sn[j] : L.sin_t[(size_t)pos * half + c];
+                rotate_pair(x1, x2, cs, sn, o1, o2);
+              }
               if (head < nq) {
-                bf16_t* dst = a.q + (size_t)token * (nq * D) + (size_t)head * D + c;
+                bf16_t* dst = qbuf + (size_t)token * (nq * D) + (size_t)head * D + c;
                 shared_store16(dst, bf16_bits(o1));
                 shared_store16(dst + half, bf16_bits(o2));
               } else if (head < nq + nkv) {
@@ -440,137 +657,105 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
             }
           });
     }
-    mark();
+    mark(12);
     grid_barrier(gs, false);
-    mark();
+    mark(13);
 
     // ---- 2. attention of every (request, kv head) over its pages, the keys cut into splits
     {
       AttnArgs at;
-      at.q = a.q; at.q_stride = nq * D; at.out = nullptr; at.out_stride = 0;
+      at.q = qbuf; at.q_stride = nq * D; at.out = nullptr; at.out_stride = 0;
       at.kcache = L.kcache; at.vcache = L.vcache;
       at.block_table = table; at.table_stride = table_stride;
       at.q_start = nullptr; at.kv_len = a.kv_len; at.tile_req = nullptr; at.tile_row0 = nullptr; at.tile_row1 = nullptr;
       at.n_tiles = M; at.nq = nq; at.nkv = nkv; at.group = group; at.P = P; at.window = L.window;
       at.p_shift = 31 - __builtin_clz(P);
       at.scale_log2 = a.scale * 1.4426950408889634f;
-      at.split = a.split; at.max_splits = a.max_splits; at.part_o = a.part_o; at.part_ml = a.part_ml;
+      at.split = a.split; at.max_splits = a.max_splits; at.part_o = part_o; at.part_ml = part_ml;
       const int n_items = M * nkv * a.max_splits;
       for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
         const int split_index = item % a.max_splits, rest = item / a.max_splits;
         attention_item<DT, 1, BIG, true>(at, rest / nkv, rest % nkv, split_index, lds, DL_WAVES);
         __syncthreads();  // the next item uses the same LDS
       }
+      mark(21);
+      // the output product's weights: on their way through the barrier (the attention itself
+      // leaves no registers to hold them any earlier)
+      w_o.begin(L.w_o, zeros, nq * D, H, 0, 0, wave, r, q);
     }
-    mark();
+    mark(22);
     grid_barrier(gs, false);
-    mark();
+    mark(23);
 
     // ---- 3. xb = x + attention * Wo^T; the attention's splits are merged on the way in
-    product_phase<false>(
-        L.w_o, nq * D, H, 0, 0, lds,
-        [&](int step, bool) -> bf16x8_t {
-          const int k0 = step * 32 + q * 8;
-          if (r >= M || k0 >= nq * D) return dl_zero8();
-          const int head = k0 / D, c0 = k0 - head * D;
-          const int kvh = head / group, row = head - kvh * group;
-          const int kvl = a.kv_len[r];
-          const int lo = L.window > 0 ? max(0, kvl - L.window) : 0;
-          const int s_first = lo / a.split, nsp = (kvl - 1) / a.split - s_first + 1;
-          const size_t item0 = ((size_t)r * nkv + kvh) * a.max_splits;
-          const float* ml = a.part_ml + (item0 * 16 + row) * 2;
-          const float* po = a.part_o + (item0 * 16 + row) * D + c0;
-          float m = -INFINITY;
-          for (int sp = 0; sp < nsp; ++sp) {
-            union { uint64_t u; float f[2]; } v;
-            v.u = shared_load64(ml + (size_t)sp * 32);
-            m = fmaxf(m, v.f[0]);
-          }
-          float l = 0.f, o[8];
+    {
+      bf16_t* stage = (bf16_t*)(lds + DL_SSQ_FLOATS + DL_RED_FLOATS);
+      merge_attention<D>(a, part_o, part_ml, L.window, stage);
+      __syncthreads();
+      mark(29);
+      // the gate | up weights, the largest of a block: on their way through this product and the barrier behind it
+      w_gu.begin(L.w_gu, zeros, H, I, 0, I, wave, r, q);
+      product_run(
+          w_o, lds, mark, 30, r, q,
+          [&](int step, bool) { return *(const bf16x8_t*)(stage + (size_t)(min(step, (nq * D + 31) / 32 - 1) * 64 + lane) * 8); },
+          [&]() {},
+          [&](int token, int, int unit0, int limit, f32x4_t s0, f32x4_t) {
+            if (token >= M) return;
+            float o[4], res[4];
+            load_row4(x_in + (size_t)token * H, unit0, limit, res);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) o[e] = 0.f;
-          for (int sp = 0; sp < nsp; ++sp) {
-            union { uint64_t u; float f[2]; } v;
-            v.u = shared_load64(ml + (size_t)sp * 32);
-            const float w = v.f[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(v.f[0] - m);
-            l += w * v.f[1];
-            const float* src = po + (size_t)sp * 16 * D;
-#pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-              union { uint64_t u; float f[2]; } pv;
-              pv.u = shared_load64(src + e);
-              o[e] += w * pv.f[0];
-              o[e + 1] += w * pv.f[1];
-            }
-          }
-          const float inv = 1.0f / l;
-          bf16x8_t out;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) out[e] = (__bf16)(o[e] * inv);
-          return out;
-        },
-        [&]() {},
-        [&](int token, int, int unit0, int limit, f32x4_t s0, f32x4_t) {
-          if (token >= M) return;
-          float o[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            o[j] = 0.f;
-            if (unit0 + j < limit) {
-              union { uint16_t u; } res;
-              // the residual is this workgroup's own slice of x, but written by another phase's workgroups
-              res.u = __hip_atomic_load((const uint16_t*)(a.x + (size_t)token * H + unit0 + j), __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_AGENT);
-              o[j] = round_to<bf16_t>(s0[j]) + bf16_bits_to_f32(res.u);
-            }
-          }
-          store_row4(a.xb + (size_t)token * H, unit0, limit, o);
-        });
-    mark();
+            for (int j = 0; j < 4; ++j) o[j] = round_to<bf16_t>(s0[j]) + res[j];
+            store_row4(xb + (size_t)token * H, unit0, limit, o);
+          });
+    }
+    mark(32);
     grid_barrier(gs, false);
-    mark();
+    mark(33);
 
     // ---- 4. h = silu(gate) * up of the normed stream
     {
       float ssq = 0.f;
-      product_phase<true>(
-          L.w_gu, H, I, 0, I, lds,
-          [&](int step, bool first) { return load_normed(a.xb, H, M, L.norm2, L.norm2_f32, step, r, q, first, ssq); },
-          [&]() { put_ssq(lds, ssq, wave, lane); },
+      product_run(
+          w_gu, lds, mark, 40, r, q,
+          [&](int step, bool first) { return load_normed(xb, zeros, H, M, L.norm2, L.norm2_f32, step, r, q, first, ssq); },
+          [&]() {
+            put_ssq(lds, ssq, wave, lane);
+            w_down.begin(L.w_down, zeros, I, H, 0, 0, wave, r, q);  // the down product's weights: on their way through the barrier
+          },
           [&](int token, int, int unit0, int limit, f32x4_t s0, f32x4_t s1) {
             if (token >= M) return;
             const float rstd = rstd_of(lds, token, H, L.eps2);
             float o[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) o[j] = silu_mul_bf16(s0[j] * rstd, s1[j] * rstd);
-            store_row4(a.h + (size_t)token * I, unit0, limit, o);
+            store_row4(hbuf + (size_t)token * I, unit0, limit, o);
           });
     }
-    mark();
+    mark(42);
     grid_barrier(gs, false);
-    mark();
+    mark(43);
 
     // ---- 5. x = xb + h * Wdown^T (and, after the last block, what the following norm needs)
     {
-      float* emit_part = lds + DL_SSQ_FLOATS + DL_MAX_TILES * DL_WAVES * 64 * 4;  // [tile * 4 + quarter][16 tokens], behind the sums
+      float* emit_part = lds + DL_SSQ_FLOATS + DL_RED_FLOATS;  // [tile * 4 + quarter][16 tokens], behind the sums
       const bool emit = last_layer && a.emit_w != nullptr;
-      const PhaseShape shape = phase_shape(H);
-      product_phase<false>(
-          L.w_down, I, H, 0, 0, lds,
-          [&](int step, bool) { return load_rows(a.h, I, M, I, step, r, q); },
-          [&]() {},
+      const PhaseShape shape = w_down.s.p;
+      product_run(
+          w_down, lds, mark, 50, r, q,
+          [&](int step, bool) { return load_rows(hbuf, zeros, I, M, I, step, r, q); },
+          [&]() {
+            // the next block's q | k | v weights: on their way through the barrier
+            if (!last_layer) w_qkv.begin(a.layers[li + 1].w_qkv, zeros, H, (nq + 2 * nkv) * half, half, half, wave, r, q);
+          },
           [&](int token, int slot, int unit0, int limit, f32x4_t s0, f32x4_t) {
-            float o[4], ss = 0.f;
+            float o[4] = {0.f, 0.f, 0.f, 0.f}, ss = 0.f;
+            if (token < M) {
+              float res[4];
+              load_row4(xb + (size_t)token * H, unit0, limit, res);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              o[j] = 0.f;
-              if (token < M && unit0 + j < limit) {
-                const uint16_t res = __hip_atomic_load((const uint16_t*)(a.xb + (size_t)token * H + unit0 + j),
-                                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                o[j] = round_to<bf16_t>(s0[j]) + bf16_bits_to_f32(res);
-              }
+              for (int j = 0; j < 4; ++j) o[j] = round_to<bf16_t>(s0[j]) + res[j];
+              store_row4(x_out + (size_t)token * H, unit0, limit, o);
             }
-            if (token < M) store_row4(a.x + (size_t)token * H, unit0, limit, o);
             if (emit) {
               float sc[4];
 #pragma unroll
@@ -600,20 +785,23 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
         }
       }
     }
-    mark();
+    mark(52);
     grid_barrier(gs, last_layer);
-    mark();
+    mark(53);
   }
 }
 
 // ---------------------------------------------------------------------------------
 // launch
 // ---------------------------------------------------------------------------------
-static size_t decode_lds_bytes(int d) {
-  const size_t product = sizeof(float) * (DL_SSQ_FLOATS + (size_t)2 * DL_MAX_TILES * DL_WAVES * 64 * 4);
-  const size_t emit = sizeof(float) * (DL_SSQ_FLOATS + (size_t)DL_MAX_TILES * DL_WAVES * 64 * 4 + DL_MAX_TILES * 4 * 16);
+static size_t decode_lds_bytes(int d, int nq) {
+  const size_t product = sizeof(float) * (DL_SSQ_FLOATS + (size_t)2 * DL_RED_FLOATS);
+  const size_t emit = sizeof(float) * (DL_SSQ_FLOATS + (size_t)DL_RED_FLOATS + DL_MAX_TILES * 4 * 16);
+  // the output product: its sums, and behind them the merged attention, 1 KB a step of 32
+  const size_t merged = sizeof(float) * (DL_SSQ_FLOATS + (size_t)DL_RED_FLOATS) + (size_t)((nq * d + 31) / 32) * 1024;
   const size_t attention = sizeof(float) * (size_t)DL_WAVES * 16 * (d + 4);
   size_t n = product > emit ? product : emit;
+  n = n > merged ? n : merged;
   return n > attention ? n : attention;
 }
 
@@ -627,7 +815,7 @@ static int decode_groups() {
 
 template <int DT>
 static bool launch_decode(const DecodeArgs& a, int groups, hipStream_t stream) {
-  const size_t lds = decode_lds_bytes(DT * 16);
+  const size_t lds = decode_lds_bytes(DT * 16, a.nq);
   auto kernel = a.P >= 16 ? decode_layers_kernel<DT, true> : decode_layers_kernel<DT, false>;
   if (lds > 64 * 1024 &&
       hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -647,7 +835,7 @@ static int decode_check(int M, int H, int I, int nq, int nkv, int d, int P, int 
   TK_REQUIRE(M >= 1 && M <= 16, "decode_layers: %d tokens, the kernel takes 1 to 16", M);
   TK_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0 && nq / nkv <= 16,
              "decode_layers: %d query heads over %d kv heads (at most 16 a kv head)", nq, nkv);
-  TK_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "decode_layers: head size %d is not a multiple of 16 up to 128", d);
+  TK_REQUIRE(d == 16 || d == 32 || d == 64 || d == 128, "decode_layers: head size %d is not 16, 32, 64 or 128", d);
   TK_REQUIRE(P >= 4 && (P & (P - 1)) == 0, "decode_layers: page size %d is not a power of two from 4", P);
   TK_REQUIRE(H > 0 && I > 0 && H % 8 == 0 && I % 8 == 0, "decode_layers: widths %d and %d must be multiples of 8", H, I);
   TK_REQUIRE(groups >= 1 && groups <= DL_MAX_GROUPS, "decode_layers: %d workgroups", groups);
@@ -656,6 +844,7 @@ static int decode_check(int M, int H, int I, int nq, int nkv, int d, int P, int 
   for (int i = 0; i < 4; ++i)
     TK_REQUIRE((units[i] + groups - 1) / groups <= limit,
                "decode_layers: %d outputs over %d workgroups are more than %d each", units[i], groups, limit);
+  TK_REQUIRE(decode_lds_bytes(d, nq) <= 160 * 1024, "decode_layers: %d heads of size %d do not fit the local memory", nq, d);
   return 0;
 }
 
@@ -676,27 +865,27 @@ TK_API int tk_decode_layers(const DecodeArgs* args, int groups, hipStream_t stre
   TK_REQUIRE(groups > 0, "decode_layers: the device's compute units could not be counted");
   if (decode_check(a.M, a.H, a.I, a.nq, a.nkv, a.d, a.P, groups) != 0) return -1;
   TK_REQUIRE(a.n_layers >= 0 && (a.n_layers == 0 || a.layers != nullptr), "decode_layers: no layers");
-  TK_REQUIRE(a.positions && a.kv_len && a.x && a.xb && a.q && a.h && a.part_o && a.part_ml && a.sync && a.status,
+  TK_REQUIRE(a.positions && a.kv_len && a.xs && a.xbs && a.qs && a.hs && a.part_o && a.part_ml && a.sync && a.status,
              "decode_layers: an operand is missing");
-  TK_REQUIRE(a.split > 0 && a.split % (32 * DL_WAVES) == 0 && a.max_splits >= 1,
-             "decode_layers: a split of %d keys is no multiple of %d", a.split, 32 * DL_WAVES);
+  TK_REQUIRE(a.split > 0 && a.split % (32 * DL_WAVES) == 0 && a.max_splits >= 1 && a.max_splits <= DL_MAX_SPLITS,
+             "decode_layers: a split of %d keys is no multiple of %d, or %d splits are more than %d", a.split, 32 * DL_WAVES,
+             a.max_splits, DL_MAX_SPLITS);
   TK_REQUIRE(a.scale > 0.f, "decode_layers: the scale must be positive");
-  TK_REQUIRE((((uintptr_t)a.x | (uintptr_t)a.xb | (uintptr_t)a.q | (uintptr_t)a.h | (uintptr_t)a.part_o |
+  TK_REQUIRE((((uintptr_t)a.xs | (uintptr_t)a.xbs | (uintptr_t)a.qs | (uintptr_t)a.hs | (uintptr_t)a.part_o |
                (uintptr_t)a.part_ml) & 15) == 0, "decode_layers: operands must be 16-byte aligned");
   TK_REQUIRE(a.emit_w == nullptr || (a.emit_scaled && a.emit_sumsq), "decode_layers: outputs for the following norm are missing");
   TK_REQUIRE(a.spin_cap > 0, "decode_layers: the spin limit must be positive");
   if (a.expect_groups == 0) a.expect_groups = (uint32_t)groups;
   if (a.n_layers == 0) return 0;
+  // built for the head sizes 16, 32, 64 and 128 (each instance is a large kernel); others are
+  // refused by tk_decode_layers_supports and run through the separate kernels
   bool ok;
   switch (a.d / 16) {
     case 1: ok = launch_decode<1>(a, groups, stream); break;
     case 2: ok = launch_decode<2>(a, groups, stream); break;
-    case 3: ok = launch_decode<3>(a, groups, stream); break;
     case 4: ok = launch_decode<4>(a, groups, stream); break;
-    case 5: ok = launch_decode<5>(a, groups, stream); break;
-    case 6: ok = launch_decode<6>(a, groups, stream); break;
-    case 7: ok = launch_decode<7>(a, groups, stream); break;
-    default: ok = launch_decode<8>(a, groups, stream); break;
+    case 8: ok = launch_decode<8>(a, groups, stream); break;
+    default: TK_REQUIRE(false, "decode_layers: no kernel was built for head size %d", a.d);
   }
   TK_REQUIRE(ok, "decode_layers: the kernel's local memory could not be reserved");
   TK_CHECK_LAUNCH("decode_layers");

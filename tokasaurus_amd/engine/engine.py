@@ -101,6 +101,7 @@ class Engine:
             )
         else:
             config.finalize(runner.max_positions)
+        runner.model.fuse_decode = bool(config.fuse_decode_layers)
         self.runner = runner
         limit = config.max_num_tokens_per_request or runner.max_positions
         self.scheduler = Scheduler(

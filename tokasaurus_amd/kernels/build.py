@@ -1,9 +1,10 @@
 """Builds the gfx950 kernel libraries from ``tokasaurus_amd/csrc`` with hipcc.
 
-There are two shared objects, loaded through ctypes (no Python headers, no torch
+There are three shared objects, loaded through ctypes (no Python headers, no torch
 headers): ``core`` holds the kernels every model needs in either storage type,
 ``mfma`` the bfloat16 matrix-core kernels, which a 32-bit run never loads and so
-never compiles.  A fresh checkout builds what it needs at its first call in
+never compiles, ``fused`` the run of blocks in one kernel, which only an engine that
+is told to use it loads.  A fresh checkout builds what it needs at its first call in
 well under a minute.  ``ensure_built`` is what the loader calls: it compiles only
 when no library matching the current sources exists, and prints a line per file
 meanwhile.  The libraries live in ``tokasaurus_amd/kernels/_build``; when that
@@ -27,7 +28,9 @@ CSRC = Path(__file__).resolve().parent.parent / "csrc"
 IN_TREE_DIR = Path(__file__).resolve().parent / "_build"
 GROUPS = {
     "core": ["errors.hip", "elementwise.hip", "attention_generic.hip", "gemm_generic.hip", "sample.hip"],
-    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip", "decode_layers.hip"],
+    "mfma": ["errors.hip", "attention_mfma.hip", "gemm_mfma.hip"],
+    # the run of blocks in one kernel: large, and only loaded when an engine is told to use it
+    "fused": ["errors.hip", "decode_layers.hip"],
 }
 
 ARCH = "gfx950"
@@ -52,6 +55,12 @@ SOURCE_FLAGS = {"attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
                 "decode_layers.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
 
+# A developer's knob: extra flags for every hipcc call (for instance -DDL_ONLY_DT=4 builds the
+# run-of-blocks kernel for one head size only, in a fraction of the time).  Part of the digest,
+# so a library built with it is not taken for one built without.
+EXTRA_FLAGS = os.environ.get("TOKASAURUS_HIPCC_EXTRA", "").split()
+
+
 class BuildError(RuntimeError):
     pass
 
@@ -69,7 +78,7 @@ def _hipcc() -> str:
 
 def _digest(group: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + EXTRA_FLAGS).encode())
     h.update(repr(sorted(SOURCE_FLAGS.items())).encode())
     for p in sorted(CSRC.glob("*.h")) + sources(group):
         h.update(p.name.encode())
@@ -121,7 +130,7 @@ def _say(msg: str) -> None:
 
 def _compile_one(hipcc: str, src: Path, obj: Path) -> tuple[Path, float]:
     t0 = time.time()
-    cmd = [hipcc, *HIPCC_FLAGS, *SOURCE_FLAGS.get(src.name, []), "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS, *SOURCE_FLAGS.get(src.name, []), "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise BuildError(f"hipcc failed on {src.name}:\n{proc.stderr[-4000:]}")

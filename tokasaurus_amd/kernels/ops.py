@@ -772,9 +772,12 @@ def add(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
 # a run of blocks in one kernel (decode steps of few tokens)
 # --------------------------------------------------------------------------
 
+# Experimental and off unless an engine is told otherwise (EngineConfig.fuse_decode_layers): on an
+# MI355X the run is correct in every cutting but slower than the separate kernels so far.
 DECODE_LAYERS_ROWS = 16  # tokens the kernel takes (one a request)
 DECODE_LAYERS_WAVES = 8  # wavefronts of its workgroups: a split of the keys is a multiple of 32 times this
 DECODE_LAYERS_TABLES = 4  # block tables (cache groups) one run may use
+DECODE_MARKS_PER_LAYER = 24  # timing marks a block may leave (DL_MARKS_PER_LAYER)
 DECODE_SPIN_CAP = 2_000_000  # polls a workgroup waits at a barrier before it gives up (seconds, not microseconds)
 
 
@@ -798,7 +801,7 @@ class _DecodeArgs(ctypes.Structure):
         ("d", ctypes.c_int), ("P", ctypes.c_int),
         ("positions", ctypes.c_void_p), ("kv_len", ctypes.c_void_p),
         ("tables", ctypes.c_void_p * DECODE_LAYERS_TABLES), ("table_stride", ctypes.c_int * DECODE_LAYERS_TABLES),
-        ("x", ctypes.c_void_p), ("xb", ctypes.c_void_p), ("q", ctypes.c_void_p), ("h", ctypes.c_void_p),
+        ("xs", ctypes.c_void_p), ("xbs", ctypes.c_void_p), ("qs", ctypes.c_void_p), ("hs", ctypes.c_void_p),
         ("part_o", ctypes.c_void_p), ("part_ml", ctypes.c_void_p), ("split", ctypes.c_int), ("max_splits", ctypes.c_int),
         ("scale", ctypes.c_float),
         ("emit_w", ctypes.c_void_p), ("emit_w_f32", ctypes.c_int), ("emit_scaled", ctypes.c_void_p), ("emit_sumsq", ctypes.c_void_p),
@@ -836,7 +839,7 @@ class DecodeLayerSpec:
 
 def decode_layers_supports(m: int, hidden: int, inter: int, nq: int, nkv: int, head_dim: int, page_size: int) -> bool:
     """Whether the one-kernel run takes these sizes on the current device."""
-    lib = load("mfma")
+    lib = load("fused")
     return lib.tk_decode_layers_supports(m, hidden, inter, nq, nkv, head_dim, page_size) == 0
 
 
@@ -850,7 +853,7 @@ def decode_sync(device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
     if key not in _decode_sync:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("decode_layers: the barrier's memory must exist before a step is recorded")
-        words = load("mfma").tk_decode_layers_sync_words()
+        words = load("fused").tk_decode_layers_sync_words()
         _decode_sync[key] = (torch.zeros((words,), dtype=torch.int32, device=device),
                              torch.zeros((1,), dtype=torch.int32, device=device))
     return _decode_sync[key]
@@ -892,7 +895,7 @@ class DecodeLayers:
         self.page_size = page_size
         self.specs = specs
         self.device = first.w_qkv.device
-        lib = load("mfma")
+        lib = load("fused")
         _need(lib.tk_decode_layers_layer_bytes() == ctypes.sizeof(_DecodeLayer), "decode_layers: struct DecodeLayer differs between library and wrapper")
         tables: list[int] = []  # distinct block tables in order of first use (by the tensor's identity)
         arr = (_DecodeLayer * len(specs))()
@@ -959,12 +962,14 @@ def decode_layers(
 ):
     """The blocks of ``run`` on the rows of ``x`` [M <= 16, H] (one token a request, request r
     at ``positions[r]`` holding ``kv_len[r]`` keys after this step), in one kernel.  Returns the
-    new residual stream (``x`` itself, overwritten) and, with ``emit_weight`` (the weight of the
+    new residual stream and, with ``emit_weight`` (the weight of the
     RMSNorm that follows), the ``Prenorm`` record for the product behind that norm.
     ``block_tables``: for every block of the run its cache group's table [M, width].
     ``kv_bound`` bounds kv_len: it cuts the keys into splits, whatever the lengths are.
-    ``timing`` (int64 [1 + 10 * blocks], diagnostics): workgroup ``timing_group`` leaves the
-    100 MHz clock at its start and after every phase and every barrier of every block."""
+    ``timing`` (int64 [2 * (1 + DECODE_MARKS_PER_LAYER * blocks)], diagnostics): workgroup
+    ``timing_group`` leaves pairs (mark, 100 MHz clock) at its start and at the ends of the parts
+    of every phase of every block (marks 10.. q|k|v, 20.. attention, 30.. output product,
+    40.. gate|up, 50.. down; x2 a phase's end, x3 the end of the barrier behind it)."""
     _gpu(x, positions, kv_len, emit_weight, *block_tables)
     m = x.shape[0]
     _need(x.dim() == 2 and x.shape[1] == run.hidden and x.dtype == torch.bfloat16 and x.is_contiguous(),
@@ -983,17 +988,21 @@ def decode_layers(
         _need(seen.setdefault(idx, t) is t or seen[idx].data_ptr() == t.data_ptr(), "decode_layers: the blocks of one cache group must bring one table")
         args.tables[idx] = t.data_ptr()
         args.table_stride[idx] = t.stride(0)
-    lib = load("mfma")
+    lib = load("fused")
     groups = lib.tk_decode_layers_groups()
     split, max_splits = decode_split(kv_bound, m, run.nkv, groups)
     dev = x.device
     sync, status = decode_sync(dev)
-    xb = torch.empty_like(x)
-    q = torch.empty((m, run.nq * run.d), dtype=torch.bfloat16, device=dev)
-    h = torch.empty((m, run.inter), dtype=torch.bfloat16, device=dev)
+    # every block has scratch of its own: within a launch a buffer is written once
+    n = len(run.specs)
+    xs = torch.empty((n + 1, m, run.hidden), dtype=torch.bfloat16, device=dev)
+    xs[0].copy_(x)
+    xbs = torch.empty((n, m, run.hidden), dtype=torch.bfloat16, device=dev)
+    qs = torch.empty((n, m, run.nq * run.d), dtype=torch.bfloat16, device=dev)
+    hs = torch.empty((n, m, run.inter), dtype=torch.bfloat16, device=dev)
     items = m * run.nkv * max_splits * 16
-    part_o = torch.empty((items * run.d,), dtype=torch.float32, device=dev)
-    part_ml = torch.empty((items * 2,), dtype=torch.float32, device=dev)
+    part_o = torch.empty((n * items * run.d,), dtype=torch.float32, device=dev)
+    part_ml = torch.empty((n * items * 2,), dtype=torch.float32, device=dev)
     emitted = None
     if emit_weight is not None:
         _need(emit_weight.shape == (run.hidden,) and emit_weight.is_contiguous() and emit_weight.dtype in (torch.bfloat16, torch.float32),
@@ -1005,15 +1014,21 @@ def decode_layers(
     args.layers, args.n_layers = run.layers.data_ptr(), len(run.specs)
     args.M, args.H, args.I, args.nq, args.nkv, args.d, args.P = m, run.hidden, run.inter, run.nq, run.nkv, run.d, run.page_size
     args.positions, args.kv_len = positions.data_ptr(), kv_len.data_ptr()
-    args.x, args.xb, args.q, args.h = x.data_ptr(), xb.data_ptr(), q.data_ptr(), h.data_ptr()
+    args.xs, args.xbs, args.qs, args.hs = xs.data_ptr(), xbs.data_ptr(), qs.data_ptr(), hs.data_ptr()
     args.part_o, args.part_ml, args.split, args.max_splits = part_o.data_ptr(), part_ml.data_ptr(), split, max_splits
     args.scale = run.scale
     args.sync, args.status = sync.data_ptr(), status.data_ptr()
     args.spin_cap, args.expect_groups = int(spin_cap), int(expect_groups)
     if timing is not None:
         _gpu(timing)
-        _need(timing.dtype == torch.int64 and timing.is_contiguous() and timing.numel() >= 1 + 10 * len(run.specs),
-              "decode_layers: timing must be int64 [1 + 10 * blocks]")
+        _need(timing.dtype == torch.int64 and timing.is_contiguous()
+              and timing.numel() >= 2 * (1 + DECODE_MARKS_PER_LAYER * len(run.specs)),
+              "decode_layers: timing must be int64 [2 * (1 + DECODE_MARKS_PER_LAYER * blocks)]")
         args.timing, args.timing_group = timing.data_ptr(), int(timing_group)
     call("tk_decode_layers", ctypes.byref(args), 0, _stream())
-    return x, emitted
+    global decode_layers_calls
+    decode_layers_calls += 1
+    return xs[n], emitted
+
+
+decode_layers_calls = 0  # launches so far (tests ask whether a step went this way)

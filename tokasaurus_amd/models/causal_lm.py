@@ -26,8 +26,8 @@ class CausalLM:
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self.weight_bytes = 0
-        # decode steps of few tokens run neighbouring blocks that allow it in one kernel
-        # (kernels.ops.decode_layers); False: every block launches its own kernels
+        # True: decode steps of few tokens run neighbouring blocks that allow it in one kernel
+        # (kernels.ops.decode_layers, experimental); False: every block launches its own kernels
         self.fuse_decode = False
         self._decode_runs: dict = {}
 
