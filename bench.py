@@ -65,6 +65,8 @@ def parse() -> argparse.Namespace:
     p.add_argument("--prefill-only", action="store_true", help="time only the prefill (for profiles); prints its record alone")
     p.add_argument("--eager", action="store_true", help="no HIP graphs")
     p.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes (the default is the headline's)")
+    p.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                   help="instead of the decode steps: a whole workload through Engine.generate (prints its own line)")
     return p.parse_args()
 
 
@@ -75,6 +77,76 @@ LLAMA_8B = dict(LLAMA_1B, num_hidden_layers=32, hidden_size=4096, num_attention_
                 intermediate_size=14336, tie_word_embeddings=False,
                 rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=8.0))
 SHAPES = {"1b": ("llama-3.2-1b-shape", LLAMA_1B), "3b": ("llama-3.2-3b-shape", LLAMA_3B), "8b": ("llama-3.1-8b-shape", LLAMA_8B)}
+
+
+# The two serving workloads the reference's numbers are quoted on, with seeded random token ids
+# of the stated lengths in place of the data sets (tokasaurus/logs/blog_commands.md:41-43).
+WORKLOADS = {
+    # 64 sequences, prompts uniform in [128, 4096], 512 decode tokens each
+    "3b-mixed": dict(shape="3b", seqs=64, prompt=(128, 4096), decode=512, max_tokens_per_forward=8192, graph_max=128),
+    # 256 concurrent sequences of 1 024 prompt and 1 024 decode tokens under max_tokens_per_forward 8192
+    "8b-concurrent": dict(shape="8b", seqs=256, prompt=(1024, 1024), decode=1024, max_tokens_per_forward=8192, graph_max=256),
+}
+
+
+def run_workload(args) -> int:
+    """Every sequence submitted at once, the engine schedules (prompt portions beside decoding
+    under the token budget); prints total, prompt and decode tokens a second and the stats line."""
+    import torch
+
+    from tokasaurus_amd.config import EngineConfig
+    from tokasaurus_amd.engine.engine import Engine
+    from tokasaurus_amd.engine.runner import ModelRunner
+    from tokasaurus_amd.sampling import SamplingParams
+
+    w = WORKLOADS[args.workload]
+    model_name, shape = SHAPES[w["shape"]]
+    cfgd = dict(shape)
+    g = torch.Generator().manual_seed(0)
+    lo, hi = w["prompt"]
+    lengths = [int(torch.randint(lo, hi + 1, (1,), generator=g)) for _ in range(w["seqs"])]
+    per_request = hi + w["decode"]
+    tokens = -(-sum(n + w["decode"] for n in lengths) // PAGE_SIZE) * PAGE_SIZE + w["seqs"] * PAGE_SIZE
+    runner = ModelRunner.from_random(cfgd, 0, args.dtype, PAGE_SIZE, tokens // PAGE_SIZE, w["seqs"],
+                                     max_tokens_per_request=per_request, use_graphs=not args.eager, graph_max_size=w["graph_max"])
+    cfg = EngineConfig(dtype=args.dtype, page_size=PAGE_SIZE, kv_cache_num_tokens=tokens,
+                       max_tokens_per_forward=w["max_tokens_per_forward"], max_seqs_per_forward=w["seqs"],
+                       use_hipgraphs=not args.eager, hipgraph_max_size=w["graph_max"], stats_report_seconds=0)
+    engine = Engine(cfg, runner=runner)
+    vocab = cfgd["vocab_size"]
+    prompts = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lengths]
+    params = SamplingParams(temperature=0.0, max_tokens=w["decode"], ignore_eos=True)
+    # one short untimed run: kernels loaded, the library's products chosen, decode steps recorded
+    engine.generate([p[:64] for p in prompts], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    engine.stats = type(engine.stats)()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    done = engine.generate(prompts, params)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    assert all(len(c.tokens) == w["decode"] for c in done)
+    st = engine.report()
+    prompt_tokens, decode_tokens = sum(lengths), w["seqs"] * w["decode"]
+    say(f"{args.workload}: {w['seqs']} sequences, {prompt_tokens} prompt and {decode_tokens} decode tokens in {seconds:.2f} s, "
+        f"{st['steps']} steps, {st['tok_per_forward']:.0f} tokens a step")
+    key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": f"total tok/s, workload {args.workload} ({model_name})",
+        "value": round((prompt_tokens + decode_tokens) / seconds, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": st["steps"], "warmup": 0, "ms_per_step": round(seconds * 1e3 / max(st["steps"], 1), 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": key,
+        "data": "synthetic (seeded random weights and token ids of the workload's lengths)",
+        "config": {"model": model_name, "global_batch": w["seqs"], "seq_len": per_request, "parallelism": "single-gpu",
+                   "layers": cfgd["num_hidden_layers"], "model_layers": cfgd["num_hidden_layers"],
+                   "hidden_size": cfgd["hidden_size"], "num_attention_heads": cfgd["num_attention_heads"],
+                   "num_key_value_heads": cfgd["num_key_value_heads"], "intermediate_size": cfgd["intermediate_size"],
+                   "vocab_size": vocab, "page_size": PAGE_SIZE, "prompt_min": lo, "prompt_max": hi, "decode_tokens": w["decode"],
+                   "max_tokens_per_forward": w["max_tokens_per_forward"], "hip_graphs": not args.eager},
+        "decode_tok_per_s": round(decode_tokens / seconds, 1), "prompt_tok_per_s": round(prompt_tokens / seconds, 1),
+        "seconds": round(seconds, 3),
+        "stats": {k: (round(v, 3) if isinstance(v, float) else v) for k, v in st.items()},
+    }))
+    return 0
 
 
 def build_runner(cfgd: dict, dtype: str, num_tokens: int, max_slots: int, context: int, use_graphs: bool):
@@ -235,6 +307,8 @@ def main() -> int:
         return 2
     import torch
 
+    if args.workload is not None:
+        return run_workload(args)
     model_name, shape = SHAPES[args.shape]
     cfgd = dict(shape)
     model_layers = cfgd["num_hidden_layers"]

@@ -45,6 +45,22 @@ def test_greedy_generation_config_a(folders):
     assert engine.runner.recorded, "decode steps were not recorded"
 
 
+def test_decode_steps_recorded_at_start_up(folders):
+    """With hipgraph_record_at_startup every size up to the live requests allowed is recorded
+    before the first request, none is recorded later for short contexts, and the completions are
+    the plain ones."""
+    cfg, _ = TINY["A"]
+    engine = engine_for(folders, "A", hipgraph_record_at_startup=True, max_seqs_per_forward=6)
+    sizes = sorted(size for size, _ in engine.runner.recorded)
+    assert sizes == [1, 2, 4, 6] or sizes == [1, 2, 4, 8], sizes
+    assert engine.runner.recorded_bytes() == sum(s * cfg["vocab_size"] * 4 for s in sizes)
+    prompts = [random_tokens(n, cfg["vocab_size"], 140 + n) for n in (5, 9, 3)]
+    done = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
+    assert sorted(size for size, _ in engine.runner.recorded) == sizes
+    for prompt, c in zip(prompts, done):
+        assert c.tokens == plain_generate(folders["A"], prompt, 6)[0]
+
+
 def test_temperature_generation_config_b_in_portions_of_16(folders):
     """Prompts of 1, 9, 70 and 130 tokens prefilled 16 tokens at a time beside the
     decoding of the others, then 12 tokens at temperature 0.8, pages of 8."""

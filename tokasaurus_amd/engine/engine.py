@@ -103,6 +103,9 @@ class Engine:
             config.finalize(runner.max_positions)
         runner.model.fuse_decode = bool(config.fuse_decode_layers)
         self.runner = runner
+        if config.use_hipgraphs and config.hipgraph_record_at_startup:
+            made = runner.record_decode_steps(max_rows=config.max_seqs_per_forward)
+            log.info("recorded %d decode steps at start-up; their outputs hold %.1f MB", made, runner.recorded_bytes() / 1e6)
         limit = config.max_num_tokens_per_request or runner.max_positions
         self.scheduler = Scheduler(
             runner.manager,

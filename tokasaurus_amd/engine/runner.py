@@ -432,6 +432,34 @@ class ModelRunner:
             self.recorded[key] = RecordedDecodeStep(self, *key)
         return self.recorded[key]
 
+    def record_decode_steps(self, max_rows: int | None = None, bounds: list[int] | None = None) -> int:
+        """Record the decode steps of every size up to ``max_rows`` (all sizes by default) for
+        the given context bounds (by default the first, 1 024 tokens, where every request
+        starts) now, instead of at their first use in the middle of a request's decoding: the
+        reference records all its sizes and warms up before it serves
+        (tokasaurus/model/utils.py:387-509,630-720).  Returns the number of recordings made;
+        each holds its own [rows, vocab] logits (and ranked tokens) in the shared pool."""
+        made = 0
+        for bound in bounds or [self.kv_bound(1)]:
+            for size in self.graph_sizes:
+                if max_rows is not None and size > max(max_rows, self.graph_sizes[0]):
+                    continue
+                key = (size, self.kv_bound(bound))
+                if key not in self.recorded:
+                    self.recorded[key] = RecordedDecodeStep(self, *key)
+                    made += 1
+        return made
+
+    def recorded_bytes(self) -> int:
+        """Memory the recordings' outputs hold (logits and ranked tokens), for the start-up log."""
+        total = 0
+        for step in self.recorded.values():
+            if step.captured:
+                total += step.logits.numel() * 4
+                if step.topk is not None:
+                    total += sum(t.numel() * 4 for t in step.topk)
+        return total
+
     def kv_bound(self, max_kv_len: int) -> int:
         """The context length a step is planned for: the power of two from 1024 that
         holds the step's longest request, at most the longest a request may get.  Parts
