@@ -549,13 +549,23 @@ __device__ __forceinline__ void merge_attention(const DecodeArgs& a, const float
   }
 }
 
+// A value the compiler must take as new: what is computed from it inside the loop over the
+// blocks stays inside that loop.  Without this the addresses and masks of every phase, which
+// do not change from block to block, are all computed ahead of the loop and kept, in far more
+// registers than a wavefront has; they come back from scratch memory in the middle of the
+// products, where every such load waits for all the weights asked for before it.
+__device__ __forceinline__ int per_block(int x) {
+  asm volatile("" : "+s"(x));
+  return x;
+}
+
 // ---------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------
 // chunks (of 8 slots) of weights a wavefront asks for ahead, per product
 #define DL_AHEAD_QKV 1
 #define DL_AHEAD_O 1
-#define DL_AHEAD_GU 2
+#define DL_AHEAD_GU 1
 #define DL_AHEAD_DOWN 2
 
 template <int DT, bool BIG>
@@ -564,8 +574,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
   constexpr int D = DT * 16;
   const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, q = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int M = a.M, H = a.H, I = a.I, nq = a.nq, nkv = a.nkv, P = a.P;
-  const int half = D / 2, group = nq / nkv;
+  constexpr int half = D / 2;
   GridSync gs = grid_sync_begin(a);
   const bf16_t* zeros = (const bf16_t*)(a.sync + 4);  // words 4 .. 7 of the sync buffer are never written
   Marks mark;
@@ -578,9 +587,11 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
   WeightStream<false, DL_AHEAD_O> w_o;
   WeightStream<true, DL_AHEAD_GU> w_gu;
   WeightStream<false, DL_AHEAD_DOWN> w_down;
-  if (a.n_layers > 0) w_qkv.begin(a.layers[0].w_qkv, zeros, H, (nq + 2 * nkv) * half, half, half, wave, r, q);
 
   for (int li = 0; li < a.n_layers; ++li) {
+    const int M = per_block(a.M), H = per_block(a.H), I = per_block(a.I), nq = per_block(a.nq), nkv = per_block(a.nkv),
+              P = per_block(a.P);
+    const int group = nq / nkv;
     const DecodeLayer L = a.layers[li];
     const int* table = a.tables[L.table];
     const int table_stride = a.table_stride[L.table];
@@ -597,6 +608,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
 
     // ---- 1. q | k | v of the normed stream, rotated; q to scratch, k and v to the pages
     {
+      w_qkv.begin(L.w_qkv, zeros, H, (nq + 2 * nkv) * half, half, half, wave, r, q);
       // what the rotation of this thread's first four units reads, asked for ahead of the product
       const PhaseShape shape = w_qkv.s.p;
       int pre_pos = 0, pre_page = 0;
@@ -679,9 +691,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
         __syncthreads();  // the next item uses the same LDS
       }
       mark(21);
-      // the output product's weights: on their way through the barrier (the attention itself
-      // leaves no registers to hold them any earlier)
-      w_o.begin(L.w_o, zeros, nq * D, H, 0, 0, wave, r, q);
     }
     mark(22);
     grid_barrier(gs, false);
@@ -690,11 +699,10 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
     // ---- 3. xb = x + attention * Wo^T; the attention's splits are merged on the way in
     {
       bf16_t* stage = (bf16_t*)(lds + DL_SSQ_FLOATS + DL_RED_FLOATS);
+      w_o.begin(L.w_o, zeros, nq * D, H, 0, 0, wave, r, q);
       merge_attention<D>(a, part_o, part_ml, L.window, stage);
       __syncthreads();
       mark(29);
-      // the gate | up weights, the largest of a block: on their way through this product and the barrier behind it
-      w_gu.begin(L.w_gu, zeros, H, I, 0, I, wave, r, q);
       product_run(
           w_o, lds, mark, 30, r, q,
           [&](int step, bool) { return *(const bf16x8_t*)(stage + (size_t)(min(step, (nq * D + 31) / 32 - 1) * 64 + lane) * 8); },
@@ -714,14 +722,12 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
 
     // ---- 4. h = silu(gate) * up of the normed stream
     {
+      w_gu.begin(L.w_gu, zeros, H, I, 0, I, wave, r, q);
       float ssq = 0.f;
       product_run(
           w_gu, lds, mark, 40, r, q,
           [&](int step, bool first) { return load_normed(xb, zeros, H, M, L.norm2, L.norm2_f32, step, r, q, first, ssq); },
-          [&]() {
-            put_ssq(lds, ssq, wave, lane);
-            w_down.begin(L.w_down, zeros, I, H, 0, 0, wave, r, q);  // the down product's weights: on their way through the barrier
-          },
+          [&]() { put_ssq(lds, ssq, wave, lane); },
           [&](int token, int, int unit0, int limit, f32x4_t s0, f32x4_t s1) {
             if (token >= M) return;
             const float rstd = rstd_of(lds, token, H, L.eps2);
@@ -739,14 +745,12 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
     {
       float* emit_part = lds + DL_SSQ_FLOATS + DL_RED_FLOATS;  // [tile * 4 + quarter][16 tokens], behind the sums
       const bool emit = last_layer && a.emit_w != nullptr;
+      w_down.begin(L.w_down, zeros, I, H, 0, 0, wave, r, q);
       const PhaseShape shape = w_down.s.p;
       product_run(
           w_down, lds, mark, 50, r, q,
           [&](int step, bool) { return load_rows(hbuf, zeros, I, M, I, step, r, q); },
-          [&]() {
-            // the next block's q | k | v weights: on their way through the barrier
-            if (!last_layer) w_qkv.begin(a.layers[li + 1].w_qkv, zeros, H, (nq + 2 * nkv) * half, half, half, wave, r, q);
-          },
+          [&]() {},
           [&](int token, int slot, int unit0, int limit, f32x4_t s0, f32x4_t) {
             float o[4] = {0.f, 0.f, 0.f, 0.f}, ss = 0.f;
             if (token < M) {
