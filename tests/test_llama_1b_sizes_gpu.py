@@ -140,3 +140,32 @@ def test_recorded_steps_with_library_products_agree_with_eager_ones(model):
     sizes = recorded_against_eager(folder, PAGE, CONFIG_1B_SIZES, 128, lengths, lambda i: 6 + (3 * i) % 23, budget=1024,
                                    padded=True)
     assert {32, 48, 64, 80, 96, 112, 128} <= sizes
+
+
+def test_sixteen_layers_deep_in_bfloat16(tmp_path):
+    """The depth of the 1B model (16 blocks, heads of 64 in groups of 4, llama3 scaling) at half its
+    width: what sixteen blocks of bfloat16 rounding add up to.  Mixed batches on few pages and the
+    last tokens one by one; every row must stay within twice the distance that the plain model
+    computing in bfloat16 keeps from the plain 32-bit logits, and the 32-bit engine within the
+    tiny models' bound."""
+    from replay_helpers import compare_with_bfloat16_measure, tail_one_by_one
+
+    cfg = dict(CONFIG_1B_SIZES, num_hidden_layers=16, hidden_size=1024, num_attention_heads=16, num_key_value_heads=4,
+               intermediate_size=2816, vocab_size=3000, max_position_embeddings=4096)
+    folder = make_folder(tmp_path / "deep", cfg, seed=8)
+    requests = {f"d{i}": random_tokens(n, cfg["vocab_size"], 700 + i) for i, n in enumerate([150, 40, 97, 64])}
+    pcfg, w = plain_llama.load_folder(folder)
+    plain = {rid: plain_llama.forward_logits(pcfg, w, toks) for rid, toks in requests.items()}
+    pcfg, w16 = plain_llama.load_folder(folder, torch.bfloat16)
+    plain16 = {rid: plain_llama.forward_logits(pcfg, w16, toks) for rid, toks in requests.items()}
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner.from_folder(folder, dtype, page_size=PAGE, num_pages=(256 + 3 * 128) // PAGE, max_slots=4)
+        got = run_steps(runner, mixed_trace(requests, seed=2))
+        got.update(run_steps(runner, tail_one_by_one("d0", requests["d0"], 32)))
+        assert len(got) == sum(len(t) for t in requests.values())
+        if dtype == "float32":
+            compare(got, plain, atol=2e-4, rtol=1e-3)  # sixteen blocks of 32-bit sums in another order
+        else:
+            worst = compare_with_bfloat16_measure(got, plain, plain16, **TOL[dtype])
+            print(f"sixteen blocks in bfloat16: at most {worst:.2f} times the plain bfloat16 model's distance")
+        assert runner.manager.num_free_pages() == [p.num_pages for p in runner.manager.pools]
