@@ -37,6 +37,7 @@
 // raises an error.  All workgroups must be resident together: the grid is at most the number of
 // compute units and a workgroup takes a compute unit's worth of wavefront slots or LDS.
 #include "attention_mfma.h"
+#include "attention_merge.h"
 
 #define DL_WAVES 8            // wavefronts of a workgroup
 #define DL_THREADS (64 * DL_WAVES)
@@ -488,67 +489,6 @@ __device__ __forceinline__ void load_row4(const bf16_t* row, int n, int limit, f
   }
 }
 
-// The attention's splits of every (token, head) merged, in split order, into the operand of
-// the output product, in LDS in the order the matrix core's lanes read it: the 8 values of
-// (step, lane = quarter * 16 + token) lie together.  All the workgroup's threads take part; the
-// partial results of up to DL_MAX_SPLITS splits are asked for at once.
-#define DL_MAX_SPLITS 16
-template <int D>
-__device__ __forceinline__ void merge_attention(const DecodeArgs& a, const float* part_o, const float* part_ml, int window,
-                                                bf16_t* stage) {
-  const int M = a.M, nq = a.nq, nkv = a.nkv, group = nq / nkv, K = nq * D;
-  const int K32 = (K + 31) >> 5;
-  // the columns past K of the last step must be zero (their weights are, and 0 * garbage may be NaN);
-  // rows of tokens past M stay as they are: they reach no output that is kept
-  for (int it = threadIdx.x; it < 16 * (K32 * 32 - K) / 4; it += DL_THREADS) {
-    const int token = it & 15, k = K + (it >> 4) * 4;
-    *(uint64_t*)(stage + ((size_t)((k >> 5) * 64 + ((k & 31) >> 3) * 16 + token) * 8 + (k & 7))) = 0;
-  }
-  const int chunks = K / 4;  // K is a multiple of 8
-  for (int it = threadIdx.x; it < M * chunks; it += DL_THREADS) {
-    const int token = it / chunks, k = (it - token * chunks) * 4;
-    union { uint64_t u; uint16_t h[4]; } pk;
-    const int head = k / D, c0 = k - head * D;
-    const int kvh = head / group, row = head - kvh * group;
-    const int kvl = a.kv_len[token];
-    const int lo = window > 0 ? max(0, kvl - window) : 0;
-    const int s_first = lo / a.split, nsp = (kvl - 1) / a.split - s_first + 1;
-    const size_t item0 = ((size_t)token * nkv + kvh) * a.max_splits;
-    const float* ml = part_ml + (item0 * 16 + row) * 2;
-    const float* po = part_o + (item0 * 16 + row) * D + c0;
-    union { uint64_t u; float f[2]; } mlv[DL_MAX_SPLITS], pa[DL_MAX_SPLITS], pb[DL_MAX_SPLITS];
-#pragma unroll
-    for (int sp = 0; sp < DL_MAX_SPLITS; ++sp) {
-      if (sp < nsp) {
-        mlv[sp].u = *(const uint64_t*)(ml + (size_t)sp * 32);
-        pa[sp].u = *(const uint64_t*)(po + (size_t)sp * 16 * D);
-        pb[sp].u = *(const uint64_t*)(po + (size_t)sp * 16 * D + 2);
-      }
-    }
-    float m = -INFINITY;
-#pragma unroll
-    for (int sp = 0; sp < DL_MAX_SPLITS; ++sp)
-      if (sp < nsp) m = fmaxf(m, mlv[sp].f[0]);
-    float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int sp = 0; sp < DL_MAX_SPLITS; ++sp) {
-      if (sp < nsp) {
-        const float w = mlv[sp].f[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mlv[sp].f[0] - m);
-        l += w * mlv[sp].f[1];
-        o[0] += w * pa[sp].f[0];
-        o[1] += w * pa[sp].f[1];
-        o[2] += w * pb[sp].f[0];
-        o[3] += w * pb[sp].f[1];
-      }
-    }
-    const float inv = 1.0f / l;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) pk.h[j] = bf16_bits(o[j] * inv);
-    const int step = k >> 5, qq = (k & 31) >> 3;
-    *(uint64_t*)(stage + ((size_t)(step * 64 + qq * 16 + token) * 8 + (k & 7))) = pk.u;
-  }
-}
-
 // A value the compiler must take as new: what is computed from it inside the loop over the
 // blocks stays inside that loop.  Without this the addresses and masks of every phase, which
 // do not change from block to block, are all computed ahead of the loop and kept, in far more
@@ -700,7 +640,10 @@ __global__ __launch_bounds__(DL_THREADS) void decode_layers_kernel(DecodeArgs a)
     {
       bf16_t* stage = (bf16_t*)(lds + DL_SSQ_FLOATS + DL_RED_FLOATS);
       w_o.begin(L.w_o, zeros, nq * D, H, 0, 0, wave, r, q);
-      merge_attention<D>(a, part_o, part_ml, L.window, stage);
+      MergeArgs mg;
+      mg.part_o = part_o; mg.part_ml = part_ml; mg.kv_len = a.kv_len;
+      mg.M = M; mg.nq = nq; mg.nkv = nkv; mg.D = D; mg.split = a.split; mg.max_splits = a.max_splits; mg.window = L.window;
+      merge_attention_to_lds(mg, stage, DL_THREADS);
       __syncthreads();
       mark(29);
       product_run(
@@ -871,9 +814,8 @@ TK_API int tk_decode_layers(const DecodeArgs* args, int groups, hipStream_t stre
   TK_REQUIRE(a.n_layers >= 0 && (a.n_layers == 0 || a.layers != nullptr), "decode_layers: no layers");
   TK_REQUIRE(a.positions && a.kv_len && a.xs && a.xbs && a.qs && a.hs && a.part_o && a.part_ml && a.sync && a.status,
              "decode_layers: an operand is missing");
-  TK_REQUIRE(a.split > 0 && a.split % (32 * DL_WAVES) == 0 && a.max_splits >= 1 && a.max_splits <= DL_MAX_SPLITS,
-             "decode_layers: a split of %d keys is no multiple of %d, or %d splits are more than %d", a.split, 32 * DL_WAVES,
-             a.max_splits, DL_MAX_SPLITS);
+  TK_REQUIRE(a.split > 0 && a.split % (32 * DL_WAVES) == 0 && a.max_splits >= 1,
+             "decode_layers: a split of %d keys is no multiple of %d", a.split, 32 * DL_WAVES);
   TK_REQUIRE(a.scale > 0.f, "decode_layers: the scale must be positive");
   TK_REQUIRE((((uintptr_t)a.xs | (uintptr_t)a.xbs | (uintptr_t)a.qs | (uintptr_t)a.hs | (uintptr_t)a.part_o |
                (uintptr_t)a.part_ml) & 15) == 0, "decode_layers: operands must be 16-byte aligned");
