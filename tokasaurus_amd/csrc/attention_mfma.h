@@ -8,20 +8,6 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-// Accesses that are coherent across the chip's dies (each has an L2 of its own): relaxed
-// atomics of agent scope, which the compiler turns into loads that go around, and stores that
-// write through, the caches.  Data that one workgroup of a running kernel writes and another
-// reads moves through these; no cache-wide write-back or invalidation is needed then.
-__device__ __forceinline__ uint64_t shared_load64(const void* p) {
-  return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void shared_store64(void* p, uint64_t v) {
-  __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void shared_store16(void* p, uint16_t v) {
-  __hip_atomic_store((uint16_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 template <bool SHARED>
 __device__ __forceinline__ bf16x8_t load_bf16x8(const bf16_t* p) {
   if constexpr (SHARED) {

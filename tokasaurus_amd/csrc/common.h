@@ -83,6 +83,20 @@ __device__ __forceinline__ float silu_mul_bf16(float g, float u) {
   return s * ur;
 }
 
+// Accesses that are coherent across the chip's dies (each has an L2 of its own): relaxed
+// atomics of agent scope, which the compiler turns into loads that go around, and stores that
+// write through, the caches.  Data that one workgroup of a running kernel writes and another
+// reads moves through these; no cache-wide write-back or invalidation is needed then.
+__device__ __forceinline__ uint64_t shared_load64(const void* p) {
+  return __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void shared_store64(void* p, uint64_t v) {
+  __hip_atomic_store((uint64_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void shared_store16(void* p, uint16_t v) {
+  __hip_atomic_store((uint16_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = TK_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, TK_WAVE);
