@@ -63,6 +63,8 @@ def parse() -> argparse.Namespace:
     p.add_argument("--points", default="1,64", help="other decode batch sizes to measure, comma separated ('' for none)")
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--prefill-only", action="store_true", help="time only the prefill (for profiles); prints its record alone")
+    p.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                   help="length of the prompt whose prefill is timed (the headline's is 2048; at most the context)")
     p.add_argument("--eager", action="store_true", help="no HIP graphs")
     p.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes (the default is the headline's)")
     p.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
@@ -322,10 +324,11 @@ def main() -> int:
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     def prefill_record(ceilings: dict | None) -> tuple[dict, dict]:
-        pdt, pstats = time_prefill(runner, PREFILL_TOKENS)
-        say(f"prefill of {PREFILL_TOKENS} tokens: mean {pstats['mean']:.2f} median {pstats['median']:.2f} min {pstats['min']:.2f} ms")
-        flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], PREFILL_TOKENS)
-        rec = {"value": round(PREFILL_TOKENS / pdt, 1), "tokens": PREFILL_TOKENS, "ms": round(pdt * 1e3, 3),
+        n = min(args.prefill_tokens, args.context)
+        pdt, pstats = time_prefill(runner, n)
+        say(f"prefill of {n} tokens: mean {pstats['mean']:.2f} median {pstats['median']:.2f} min {pstats['min']:.2f} ms")
+        flops = prefill_flops(cfgd, cfgd["num_hidden_layers"], n)
+        rec = {"value": round(n / pdt, 1), "tokens": n, "ms": round(pdt * 1e3, 3),
                "frac": round(flops / pdt / 1e12 / PEAK_TFLOPS[key], 4), "tflops": round(flops / pdt / 1e12, 1)}
         if ceilings and key == "bf16":
             rec["frac_of_measured"] = round(flops / pdt / 1e12 / ceilings["gemm_bf16_tflops"], 4)
