@@ -37,7 +37,7 @@ ATTN_CASES = [
 ]
 
 
-def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1, waves=1, pair=False):
+def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=None, row_tiles=1, waves=1, pair=False, grouped=False):
     from tokasaurus_amd.kernels import ops
 
     dtype = torch.bfloat16 if kind != "generic_f32" else torch.float32
@@ -48,7 +48,7 @@ def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=N
         token_req = torch.tensor([r for r, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32).cuda()
         positions = torch.tensor([kv - ql + j for ql, kv in zip(q_lens, kv_lens) for j in range(ql)], dtype=torch.int32).cuda()
         return ops.paged_attention_generic(q, kc, vc, table, token_req, positions, nq, nkv, d, page, window=window)
-    tile_req, tile_row0, tile_row1 = ops.attention_tiles(q_lens, nq // nkv, row_tiles, pair=pair)
+    tile_req, tile_row0, tile_row1 = ops.attention_tiles(q_lens, nq // nkv, row_tiles, pair=pair, fill=ops.ATTENTION_GROUP if grouped else 1)
     max_kv = max(kv_lens)
     if split is None:
         split, waves = ops.attention_split(max_kv, len(tile_req), nkv, d)
@@ -57,27 +57,31 @@ def run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=N
         torch.tensor(tile_req, dtype=torch.int32).cuda(), torch.tensor(tile_row0, dtype=torch.int32).cuda(),
         row_tiles, nq, nkv, d, page, max_kv, split, window=window, waves=waves,
         tile_row1=None if tile_row1 is None else torch.tensor(tile_row1, dtype=torch.int32).cuda(),
+        grouped=grouped,
     )
 
 
 @pytest.mark.parametrize("case_id", range(len(ATTN_CASES)))
 @pytest.mark.parametrize("kind", ["generic_f32", "generic_bf16", "mfma", "mfma_split32", "mfma_rt2", "mfma_rt2_waves4",
-                                  "mfma_pairs", "mfma_pairs_split32", "mfma_waves4", "mfma_waves16"])
+                                  "mfma_pairs", "mfma_pairs_split32", "mfma_waves4", "mfma_waves16", "mfma_grouped"])
 def test_paged_attention(kind, case_id):
     q_lens, kv_lens, nq, nkv, d, page, window = ATTN_CASES[case_id]
+    if kind == "mfma_grouped" and page < 16:
+        pytest.skip("tiles in groups that share their loads: pages of 16 keys or more")
     dtype = torch.float32 if kind == "generic_f32" else torch.bfloat16
     case = make_paged_case(q_lens, kv_lens, nq, nkv, d, page, seed=case_id, dtype=dtype)
     ref = attention_reference(case, q_lens, kv_lens, nq, nkv, d, window=window)
     split = {"mfma_split32": 32, "mfma_rt2": 64, "mfma_rt2_waves4": 128, "mfma_pairs": 4096, "mfma_pairs_split32": 32,
-             "mfma_waves4": 256, "mfma_waves16": 512}.get(kind)
+             "mfma_waves4": 256, "mfma_waves16": 512, "mfma_grouped": 4096}.get(kind)
     waves = {"mfma_waves4": 4, "mfma_rt2_waves4": 4, "mfma_waves16": 16}.get(kind, 1)
-    two = kind in ("mfma_rt2", "mfma_rt2_waves4", "mfma_pairs", "mfma_pairs_split32")
+    two = kind in ("mfma_rt2", "mfma_rt2_waves4", "mfma_pairs", "mfma_pairs_split32", "mfma_grouped")
     if kind.startswith("mfma"):
         from tokasaurus_amd.kernels import ops
 
         waves = min(waves, ops.attention_max_waves(d, 2 if two else 1))  # head sizes above 64 take 8 at most
     got = run_attention(kind, case, q_lens, kv_lens, nq, nkv, d, page, window, split=split,
-                        row_tiles=2 if two else 1, waves=waves, pair="pairs" in kind).float().cpu()
+                        row_tiles=2 if two else 1, waves=waves, pair="pairs" in kind,
+                        grouped=kind == "mfma_grouped").float().cpu()
     assert torch.isfinite(got).all()
     # values are of order 1; bfloat16 rounds the probabilities and the output to 8 bits
     tol = dict(atol=2e-5, rtol=1e-4) if kind == "generic_f32" else dict(atol=2e-2, rtol=2e-2)
@@ -86,7 +90,7 @@ def test_paged_attention(kind, case_id):
     assert not bad.any(), f"first wrong row {int(bad.any(1).nonzero()[0])}, largest error {float(err.max()):.3e}"
 
 
-@pytest.mark.parametrize("kind", ["generic_f32", "mfma", "mfma_pairs"])
+@pytest.mark.parametrize("kind", ["generic_f32", "mfma", "mfma_pairs", "mfma_grouped"])
 @pytest.mark.parametrize("window", [0, 600])
 def test_attention_finds_one_far_key(kind, window):
     """One key among 1,500 answers the query (its score stands out by far), the others are
@@ -110,7 +114,7 @@ def test_attention_finds_one_far_key(kind, window):
             got = run_attention(kind, case, [1], [kv_len], nq, nkv, d, page, window)
         else:
             got = run_attention(kind, case, [1], [kv_len], nq, nkv, d, page, window, split=512 if kind == "mfma" else 4096,
-                                row_tiles=2 if kind == "mfma_pairs" else 1, pair=kind == "mfma_pairs")
+                                row_tiles=1 if kind == "mfma" else 2, pair=kind == "mfma_pairs", grouped=kind == "mfma_grouped")
         got = got.float().cpu().view(nq, d)
         want = torch.stack([case["v"][0][target, h // (nq // nkv)] for h in range(nq)])
         close = torch.allclose(got, want, atol=3e-2, rtol=3e-2)

@@ -106,6 +106,43 @@ def test_mixed_batches_with_pages_used_again(folders, name, dtype):
     compare(got, ref, **TOL[dtype])
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_prompts_through_the_grouped_attention(folders, name, monkeypatch):
+    """Prompts that fill the chip several times over take an attention kernel whose workgroups
+    share every load of keys and values among four wavefronts.  Here every prompt portion of
+    more than a row tile takes it (the threshold is set to one wavefront): whole prompts,
+    portions of changing size after a past, and mixed batches of several requests on few
+    pages (groups filled up with empty tiles, tiles of different requests in one launch)."""
+    from tokasaurus_amd.kernels import ops
+
+    monkeypatch.setattr(ops, "ATTENTION_GROUPED_FROM", 1)
+    grouped_calls = 0
+    real = ops.paged_attention_mfma
+
+    def counting(*args, **kw):
+        nonlocal grouped_calls
+        grouped_calls += bool(kw.get("grouped"))
+        return real(*args, **kw)
+
+    monkeypatch.setattr(ops, "paged_attention_mfma", counting)
+    cfg, page = TINY[name]
+    lengths = [150, 80, 33, 100, 17, 260]
+    reqs = {f"g{i}": random_tokens(n, cfg["vocab_size"], 900 + i) for i, n in enumerate(lengths)}
+    ref = plain_rows(folders[name], reqs)
+    runner = runner_for(folders, name, "bfloat16", tokens=1024)
+    for rid, toks in reqs.items():
+        compare(run_steps(runner, whole(rid, toks)), ref, **TOL["bfloat16"])
+    assert grouped_calls > 0, "no launch took the grouped kernel"
+    for k, (rid, toks) in enumerate(reqs.items()):
+        sizes = [[16, 7, 2, 5, 3], [2, 2, 31, 1, 4, 9], [3, 64, 2]][k % 3]
+        compare(run_steps(runner, portions(rid, toks, sizes)), ref, **TOL["bfloat16"])
+    tokens = sum(sorted(-(-n // 64) * 64 for n in lengths)[-4:])
+    runner = runner_for(folders, name, "bfloat16", tokens=tokens)
+    got = run_steps(runner, mixed_trace(reqs, seed=5))
+    assert len(got) == sum(lengths)
+    compare(got, ref, **TOL["bfloat16"])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_and_first_tokens(folders, dtype):
     # prompt of 3, then 200 tokens one by one (crosses many pages, positions far beyond

@@ -85,7 +85,7 @@ __device__ __forceinline__ TileRange tile_range(const AttnArgs& a, int tile, int
   t.row0[1] = -1;
   if (row_tiles == 2) {
     t.row0[1] = a.tile_row1 ? a.tile_row1[tile] : t.row0[0] + 16;
-    if (t.row0[1] >= t.n_rows) t.row0[1] = -1;
+    if (t.row0[1] >= t.n_rows || t.row0[0] < 0) t.row0[1] = -1;  // row0 < 0: a tile that only fills a group
   }
   t.lo = 0x7fffffff;
   t.hi = -1;
@@ -213,9 +213,21 @@ __host__ __device__ constexpr int max_waves(int dt, int rt) { return rt == 2 ? 4
 // partial buffers, also when the tile has one split (queries are read as ever: such a kernel
 // keeps them in a buffer that is written once in a launch).
 // PF steps of loads are in flight: a lone wavefront on a long tile waits on memory otherwise.
-template <int DT, int RT, bool BIG, bool SHARED>
+// GROUPED (long prompts: two row tiles, pages of 16 keys or more, whole keys, no splits): the
+// GROUP_WAVES wavefronts of the workgroup have a tile each (`tile` is the wavefront's own, two
+// neighbouring row tiles), and all the tiles belong to one request: the host fills a request's
+// tiles up to a multiple of GROUP_WAVES with empty ones (row0 < 0).  The wavefronts walk the
+// keys that any of them sees together: every step's keys and values are loaded once, a quarter
+// by each wavefront, and pass through LDS (two buffers, one barrier a step) in the lane order
+// of the operands; the pages of a step are looked up a step before its loads are issued.  No
+// ring of loads is held in registers, so twice the wavefronts fit a SIMD, and a wavefront issues
+// a quarter of the loads and of their addresses.  wg_part: 64 bytes for the tiles' key ranges,
+// then 2 buffers of (2 KS + DT) KB.
+#define GROUP_WAVES 4
+template <int DT, int RT, bool BIG, bool SHARED, bool GROUPED = false>
 __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile, const int kvh, const int split_index,
                                                float* wg_part, const int NW) {
+  static_assert(!GROUPED || (RT == 2 && BIG && !SHARED), "grouped tiles: prompts on pages of 16 keys or more");
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head size
   constexpr int PF = RT == 1 ? 2 : 3;
@@ -223,9 +235,9 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, q = lane >> 4;
   const TileRange t = tile_range(a, tile, RT);
-  const int s = t.s_first + split_index;
-  if (s > t.s_last) return;
-  const int nsp = t.s_last - t.s_first + 1;
+  const int s = GROUPED ? 0 : t.s_first + split_index;
+  if (!GROUPED && s > t.s_last) return;
+  const int nsp = GROUPED ? 1 : t.s_last - t.s_first + 1;
   // this wavefront's part of the split: `sub` keys, a multiple of 32
   const int sub = a.split / NW;
   const int k_begin = max((t.lo >> 5) << 5, s * a.split + wave * sub);
@@ -243,18 +255,18 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
   const Range inside = range_of(t.lo, t.hi - 31);
 
   // this lane's row in each of the RT tiles
-  int pos_r[RT], lo_r[RT], flat_r[RT];
+  // (the first key a row sees and the row's number are worked out again where they are needed,
+  // at the masked steps and at the end: two registers less a row tile in the loop)
+  int pos_r[RT];
   bf16x8_t qv[RT][KS];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int flat = t.row0[rt] >= 0 ? t.row0[rt] + r : t.n_rows;
     const bool valid = flat < t.n_rows;
-    flat_r[rt] = valid ? flat : -1;
     const int fl = valid ? flat : t.n_rows - 1;
     const int tok = fl / a.group, g = fl - tok * a.group;
     const int pos = t.kvl - t.qlen + tok;
     pos_r[rt] = valid ? pos : -1;
-    lo_r[rt] = a.window > 0 ? max(0, pos - a.window + 1) : 0;
     const bf16_t* qp = a.q + (size_t)(t.qs + tok) * a.q_stride + (size_t)(kvh * a.group + g) * D;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -312,10 +324,11 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
 #pragma unroll
       for (int e = 0; e < 8; ++e) sc[e] = st[e >> 2][e & 3];
       if (!unmasked[rt].holds(kb)) {
+        const int lo_row = a.window > 0 ? max(0, pos_r[rt] - a.window + 1) : 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int key = kb + (e >> 2) * 16 + q * 4 + (e & 3);
-          if (!(key >= lo_r[rt] && key <= pos_r[rt])) sc[e] = -INFINITY;
+          if (!(key >= lo_row && key <= pos_r[rt])) sc[e] = -INFINITY;
         }
       }
       float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
@@ -346,6 +359,103 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
     }
   };
 
+  if constexpr (GROUPED) {
+    constexpr int NK = 2 * KS, NV = 2 * DT;  // fragments of a step: keys 1 KB each, values 512 bytes each
+    constexpr int NKR = (NK + GROUP_WAVES - 1) / GROUP_WAVES, NVR = (NV + GROUP_WAVES - 1) / GROUP_WAVES;
+    int* ranges = (int*)wg_part;
+    bf16x8_t* k_lds = (bf16x8_t*)(wg_part + 16);
+    bf16x4_t* v_lds = (bf16x4_t*)(k_lds + 2 * NK * 64);
+    if (lane == 0) {
+      ranges[2 * wave] = t.lo;
+      ranges[2 * wave + 1] = t.hi;
+    }
+    __syncthreads();
+    int glo = 0x7fffffff, ghi = -1;
+#pragma unroll
+    for (int w = 0; w < GROUP_WAVES; ++w) {
+      glo = min(glo, ranges[2 * w]);
+      ghi = max(ghi, ranges[2 * w + 1]);
+    }
+    glo = __builtin_amdgcn_readfirstlane(glo);
+    ghi = __builtin_amdgcn_readfirstlane(ghi);
+    if (ghi < 0) return;  // the same for every wavefront of the workgroup
+    const int g_begin = (glo >> 5) << 5, n_steps = (ghi + 1 - g_begin + 31) >> 5;
+    const int P = a.P;
+    const unsigned head_off = (unsigned)(kvh * P * D);
+    const bool mine = t.hi >= 0;  // else an empty tile: this wavefront only carries its share of the loads
+
+    bf16x8_t kreg[NKR];
+    bf16x4_t vreg[NVR];
+    // this wavefront's fragments of the step at kb, from memory into registers
+    auto fetch = [&](const int kb, const StepPages& pg) {
+#pragma unroll
+      for (int i = 0; i < NKR; ++i) {
+        const int f = i * GROUP_WAVES + wave;
+        if (f < NK) {
+          const int blk = f / KS, ks = f - blk * KS;
+          const int in_page = (kb + blk * 16) & (P - 1);
+          // (chosen, not indexed: an array indexed by a number known only at run time lives in memory)
+          const size_t base = (size_t)(unsigned)(blk ? pg.page[1] : pg.page[0]) * (unsigned)(a.nkv * P * D);
+          const int d0 = ks * 32 + q * 8;
+          if (d0 < D) {
+            kreg[i] = *(const bf16x8_t*)(a.kcache + base + head_off + (unsigned)((((d0 >> 3) * P) + in_page + r) * 8));
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) kreg[i][e] = (__bf16)0.f;
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NVR; ++i) {
+        const int f = i * GROUP_WAVES + wave;
+        if (f < NV) {
+          const int blk = f / DT, dt = f - blk * DT;
+          const int in_page = (kb + blk * 16) & (P - 1);
+          const size_t base = (size_t)(unsigned)(blk ? pg.page[1] : pg.page[0]) * (unsigned)(a.nkv * P * D);
+          vreg[i] = *(const bf16x4_t*)(a.vcache + base + head_off + (unsigned)((((in_page >> 2) + q) * (D * 4)) + (dt * 16 + r) * 4));
+        }
+      }
+    };
+    // ... from the registers into buffer `buf`
+    auto stash = [&](const int buf) {
+#pragma unroll
+      for (int i = 0; i < NKR; ++i) {
+        const int f = i * GROUP_WAVES + wave;
+        if (f < NK) k_lds[(size_t)(buf * NK + f) * 64 + lane] = kreg[i];
+      }
+#pragma unroll
+      for (int i = 0; i < NVR; ++i) {
+        const int f = i * GROUP_WAVES + wave;
+        if (f < NV) v_lds[(size_t)(buf * NV + f) * 64 + lane] = vreg[i];
+      }
+    };
+    StepPages pg = step_pages(a, table, g_begin, glo, ghi);
+    fetch(g_begin, pg);
+    if (n_steps > 1) pg = step_pages(a, table, g_begin + 32, glo, ghi);
+    stash(0);
+    if (n_steps > 1) fetch(g_begin + 32, pg);
+    if (n_steps > 2) pg = step_pages(a, table, g_begin + 64, glo, ghi);
+    __syncthreads();
+    for (int i = 0; i < n_steps; ++i) {
+      const int kb = g_begin + 32 * i, buf = i & 1;
+      // the other buffer was last read before the barrier that ended the step before
+      if (i + 1 < n_steps) stash(buf ^ 1);
+      if (i + 2 < n_steps) fetch(kb + 64, pg);
+      if (i + 3 < n_steps) pg = step_pages(a, table, kb + 96, glo, ghi);
+      if (mine && (active[0].holds(kb) || active[1].holds(kb))) {
+        StepRegs<DT> cur;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) cur.kv[blk][ks] = k_lds[(size_t)(buf * NK + blk * KS + ks) * 64 + lane];
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) cur.vv[dt].half[blk] = v_lds[(size_t)(buf * NV + blk * DT + dt) * 64 + lane];
+        }
+        compute_step(cur, kb);
+      }
+      __syncthreads();
+    }
+  } else {
   StepRegs<DT> ring[PF];
   // With two row tiles (prompts: many steps a wavefront) the pages of a step are looked up when
   // the loads of the step before are issued; with one (decode: few steps) right before its own.
@@ -370,6 +480,7 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
       }
     }
   }
+  }
 
   // acc[rt][dt][j] of lane (r, q) is O^T[d = 16 dt + 4q + j][row r]
   const size_t item0 = ((size_t)tile * a.nkv + kvh) * a.max_splits;
@@ -381,7 +492,7 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
     l_run[rt] = l;
     m_run[rt] *= a.scale_log2;  // from here on in units of log 2, as the merges take it
   }
-  if (NW > 1) {
+  if (!GROUPED && NW > 1) {
     // every wavefront leaves (max, sum, weighted values) of its rows; wavefront 0 adds them in order
     constexpr int ROW = D + 4;  // max, sum, two unused, then the values (16-byte aligned)
 #pragma unroll
@@ -418,8 +529,8 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const float l = l_run[rt];
-    const int flat = flat_r[rt];
-    if (flat < 0) continue;
+    const int flat = t.row0[rt] >= 0 ? t.row0[rt] + r : t.n_rows;
+    if (flat >= t.n_rows) continue;
     if (nsp == 1 && !SHARED) {
       const int tok = flat / a.group, g = flat - tok * a.group;
       bf16_t* op = a.out + (size_t)(t.qs + tok) * a.out_stride + (size_t)(kvh * a.group + g) * D;

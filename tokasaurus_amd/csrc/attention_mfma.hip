@@ -44,6 +44,17 @@ __global__ __launch_bounds__(64 * max_waves(DT, RT)) void paged_attention_mfma_k
   attention_item<DT, RT, BIG, false>(a, tile, kvh, blockIdx.z, wg_part, blockDim.x >> 6);
 }
 
+// Long prompts on pages of 16 keys or more: GROUP_WAVES tiles of one request a workgroup, which
+// share every load of keys and values through LDS (see attention_item, GROUPED).
+template <int DT>
+__global__ __launch_bounds__(64 * GROUP_WAVES) void paged_attention_group_kernel(AttnArgs a) {
+  extern __shared__ __align__(16) float wg_part[];
+  const int kvh = blockIdx.x % a.nkv, group = blockIdx.x / a.nkv;  // kv head fastest, as above
+  // (the wavefront's number as a scalar: what a tile covers then stays in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  attention_item<DT, 2, true, false, true>(a, group * GROUP_WAVES + wave, kvh, 0, wg_part, GROUP_WAVES);
+}
+
 // Adds the partial results of split tiles, always in split order.  One wavefront
 // per (tile, kv head, row): lane i takes the statistics of split i (of splits i, i + 64, ..),
 // then every lane sums one (or more) of the row's d outputs over the splits, with the
@@ -131,6 +142,27 @@ static bool launch_attn(const AttnArgs& a, int grid_splits, int nw, hipStream_t 
   return true;
 }
 
+template <int DT>
+static bool launch_group(const AttnArgs& a, hipStream_t stream) {
+  const size_t lds = 64 + 2 * (size_t)(2 * ((DT + 1) / 2) * 1024 + 2 * DT * 512);
+  hipLaunchKernelGGL(paged_attention_group_kernel<DT>, dim3(a.n_tiles / GROUP_WAVES * a.nkv), dim3(64 * GROUP_WAVES), lds, stream, a);
+  return true;
+}
+
+static bool launch_group_d(const AttnArgs& a, int dt, hipStream_t stream) {
+  switch (dt) {
+    case 1: return launch_group<1>(a, stream);
+    case 2: return launch_group<2>(a, stream);
+    case 3: return launch_group<3>(a, stream);
+    case 4: return launch_group<4>(a, stream);
+    case 5: return launch_group<5>(a, stream);
+    case 6: return launch_group<6>(a, stream);
+    case 7: return launch_group<7>(a, stream);
+    case 8: return launch_group<8>(a, stream);
+    default: return false;
+  }
+}
+
 template <int RT>
 static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, int nw, hipStream_t stream) {
   switch (dt) {
@@ -154,6 +186,10 @@ static bool launch_attn_d(const AttnArgs& a, int dt, int grid_splits, int nw, hi
 // max_splits).  part_o holds tiles * nkv * max_splits * 16 * row_tiles * d floats, part_ml
 // tiles * nkv * max_splits * 16 * row_tiles * 2 (both may be null when max_splits is 1).
 // Launches that share scratch must not overlap.
+// grouped != 0 (two row tiles, P >= 16, one split of whole keys, waves 1): the caller promises
+// that the tiles come in groups of 4 of one request each, filled up with empty tiles
+// (tile_row0 < 0, the request's own index in tile_req): a workgroup takes a group and loads
+// every key and value of the request's kv head once for its 4 tiles.
 TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                                        const void* kcache, const void* vcache,
                                        const int* block_table, int table_stride,
@@ -161,7 +197,7 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
                                        const int* tile_req, const int* tile_row0, const int* tile_row1,
                                        int n_tiles, int row_tiles, int nq, int nkv, int d, int P, int window,
                                        float scale, int split, int waves, int grid_splits, int max_splits,
-                                       float* part_o, float* part_ml, hipStream_t stream) {
+                                       float* part_o, float* part_ml, int grouped, hipStream_t stream) {
   TK_REQUIRE(n_tiles >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_mfma: bad sizes tiles=%d nq=%d nkv=%d", n_tiles, nq, nkv);
   TK_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attention_mfma: head size %d is not a multiple of 16 up to 128", d);
   TK_REQUIRE(P >= 4 && (P & (P - 1)) == 0, "attention_mfma: page size %d is not a power of two from 4", P);
@@ -181,6 +217,10 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
   TK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 7) == 0 && ((uintptr_t)out & 7) == 0,
              "attention_mfma: operands must be 16-byte aligned");
   TK_REQUIRE(nkv < 65536, "attention_mfma: too many kv heads");
+  TK_REQUIRE(!grouped || (row_tiles == 2 && P >= 16 && waves == 1 && max_splits == 1 && grid_splits == 1 &&
+                          n_tiles % GROUP_WAVES == 0),
+             "attention_mfma: grouped tiles need two row tiles, pages of 16 keys or more, one wavefront a tile, one split, "
+             "and a multiple of %d tiles (got %d)", GROUP_WAVES, n_tiles);
   if (n_tiles == 0) return 0;
   AttnArgs a;
   a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
@@ -192,8 +232,9 @@ TK_API int tk_paged_attention_mfma(const void* q, int q_stride, void* out, int o
   while ((1 << a.p_shift) < P) ++a.p_shift;
   a.scale_log2 = scale * 1.4426950408889634f;
   a.split = split; a.max_splits = max_splits; a.part_o = part_o; a.part_ml = part_ml;
-  const bool ok = row_tiles == 1 ? launch_attn_d<1>(a, d / 16, grid_splits, waves, stream)
-                                 : launch_attn_d<2>(a, d / 16, grid_splits, waves, stream);
+  const bool ok = grouped ? launch_group_d(a, d / 16, stream)
+                          : (row_tiles == 1 ? launch_attn_d<1>(a, d / 16, grid_splits, waves, stream)
+                                            : launch_attn_d<2>(a, d / 16, grid_splits, waves, stream));
   TK_REQUIRE(ok, "attention_mfma: no kernel for head size %d", d);
   TK_CHECK_LAUNCH("paged_attention_mfma");
   if (max_splits > 1) {

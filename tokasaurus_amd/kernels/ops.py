@@ -350,15 +350,26 @@ def check_attention_shape(dtype: torch.dtype, nq: int, nkv: int, head_dim: int, 
         call("tk_paged_attention_generic_fits", nq, nkv, head_dim)
 
 
+ATTENTION_GROUP = 4  # wavefronts (of two neighbouring row tiles each) in a workgroup of the grouped prompt kernel
+# Wavefronts (of two row tiles, over all kv heads) from which prompts take the grouped kernel: with
+# three and more a SIMD it is ahead of the kernel of paired tiles.  Measured on an MI355X, prefill
+# of one prompt, grouped against paired: 1B shape 2 048 tokens 5.85 / 5.70 ms, 4 096 tokens 10.2 /
+# 10.7 ms, 8 192 tokens 22.2 / 24.7 ms; 8B shape 4 096 tokens 51.6 / 54.3 ms, 8 192 tokens 114 / 128 ms.
+ATTENTION_GROUPED_FROM = 3072
+
+
 def attention_tiles(
-    q_lens: list[int], group: int, row_tiles: int, requests: list[int] | None = None, pair: bool = False
+    q_lens: list[int], group: int, row_tiles: int, requests: list[int] | None = None, pair: bool = False, fill: int = 1
 ) -> tuple[list[int], list[int], list[int] | None]:
     """The row tiles that cover the (token, head of the group) pairs of ``requests``
     (all by default), ``row_tiles`` tiles of 16 rows a wavefront: (request, first row of
     the first tile, first row of the second tile or -1).  With ``pair`` a request's
     i-th tile shares a wavefront with its i-th last, which evens out the keys a
     wavefront walks under a causal mask; otherwise with its neighbour, and the
-    third list is None."""
+    third list is None.  ``fill`` > 1 (two row tiles, no pairs; for the grouped kernel): a
+    request's tiles come last rows first (those that see most keys start first) and are filled
+    up to a multiple of ``fill`` with empty ones (first row -1), so that a group of ``fill``
+    never spans two requests."""
     tile_req: list[int] = []
     tile_row0: list[int] = []
     tile_row1: list[int] = []
@@ -370,9 +381,11 @@ def attention_tiles(
             firsts = [(i, n - 1 - i if n - 1 - i > i else -1) for i in range((n + 1) // 2)]
         else:
             firsts = [(i, i + 1 if i + 1 < n else -1) for i in range(0, n, 2)]
+        if fill > 1 and row_tiles == 2 and not pair:
+            firsts = firsts[::-1] + [(-1, -1)] * (-len(firsts) % fill)
         for i, j in firsts:
             tile_req.append(r)
-            tile_row0.append(16 * i)
+            tile_row0.append(16 * i if i >= 0 else -1)
             tile_row1.append(16 * j if j >= 0 else -1)
     return tile_req, tile_row0, (tile_row1 if pair and row_tiles == 2 else None)
 
@@ -451,6 +464,7 @@ def paged_attention_mfma(
     scratch: "AttentionScratch | None" = None,
     tile_row1: torch.Tensor | None = None,
     longest: int | None = None,
+    grouped: bool = False,
 ) -> torch.Tensor:
     """Attention of every token of the batch over its request's pages on the
     matrix cores (bfloat16).  ``q`` is 2-d and its first nq*d columns are the
@@ -459,7 +473,11 @@ def paged_attention_mfma(
     grid and the scratch, so it may be larger than any request's; ``longest``, if
     given, is the length of the longest request, which the block table must cover).  The tiles
     (see ``attention_tiles``) may cover some of the requests only; rows of ``out``
-    that no tile covers are left as they are."""
+    that no tile covers are left as they are.
+
+    ``grouped`` (long prompts: two neighbouring row tiles a wavefront, pages of 16 keys or more,
+    whole keys): the tiles were made with ``fill=ATTENTION_GROUP``; a workgroup takes a group of
+    them and loads the request's keys and values once for all."""
     _gpu(q, kcache, vcache, block_table, q_start, kv_len, tile_req, tile_row0)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= nq * head_dim and q.dtype == torch.bfloat16,
           "attention_mfma: q must be bfloat16, 2-d with unit inner stride and nq*d leading columns")
@@ -492,6 +510,8 @@ def paged_attention_mfma(
     else:
         _need(out.shape == (n, nq * head_dim) and out.dtype == q.dtype and out.stride(1) == 1, "attention_mfma: bad out")
     max_splits = max(1, -(-max_kv_len // split))
+    _need(not grouped or (row_tiles == 2 and page_size >= 16 and waves == 1 and max_splits == 1 and n_tiles % ATTENTION_GROUP == 0),
+          "attention_mfma: grouped tiles are prompts' (two row tiles, filled groups) on pages of 16 keys or more, unsplit")
     part_o = part_ml = None
     if max_splits > 1:
         items = n_tiles * nkv * max_splits * 16 * row_tiles
@@ -509,6 +529,7 @@ def paged_attention_mfma(
         split, waves, max_splits, max_splits,
         part_o.data_ptr() if part_o is not None else None,
         part_ml.data_ptr() if part_ml is not None else None,
+        1 if grouped else 0,
         _stream(),
     )
     return out

@@ -42,6 +42,7 @@ class AttentionLaunch:
     split: int
     waves: int
     scratch: ops.AttentionScratch | None = None  # a replayed step keeps its own
+    grouped: bool = False  # tiles in groups of one request that share their loads (long prompts)
 
 
 @dataclass
@@ -49,15 +50,17 @@ class AttentionPlan:
     """How the step's rows are cut into tiles and its keys into splits; made once
     a step for each group size and shared by the layers.  Requests that bring one
     row tile or less (decoded tokens) get wavefronts of one row tile and split keys;
-    prompt portions get wavefronts of two row tiles, an early one paired with a late
-    one, and whole keys."""
+    prompt portions get wavefronts of two row tiles and whole keys: an early tile paired with
+    a late one, or, when there are enough of them to fill the chip several times over and a
+    page holds 16 keys or more, neighbouring tiles in groups of four wavefronts that share
+    every load of keys and values."""
 
     launches: list[AttentionLaunch]
     max_kv_len: int
 
 
-def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int) -> AttentionPlan:
-    key = ("attention_plan", group, nkv, head_dim)
+def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int, page_size: int) -> AttentionPlan:
+    key = ("attention_plan", group, nkv, head_dim, page_size)
     plan = ctx.extras.get(key)
     if plan is None:
         q_lens = [ctx.host_q_start[i + 1] - ctx.host_q_start[i] for i in range(ctx.num_requests)]
@@ -66,26 +69,31 @@ def attention_plan(ctx: StepContext, group: int, nkv: int, head_dim: int) -> Att
         static = bool(ctx.extras.get("static"))
         # launches are chosen for the bound the step was planned for, not for the lengths in it
         bound = max(int(ctx.extras.get("kv_bound", 0)), ctx.max_kv_len)
-        lists: list[tuple[list[int], list[int], list[int] | None, int, int, int]] = []
+        lists: list[tuple[list[int], list[int], list[int] | None, int, int, int, bool]] = []
         if small:
             req, row0, _ = ops.attention_tiles(q_lens, group, 1, small)
             split, waves = ops.attention_split(bound, len(req), nkv, head_dim)
-            lists.append((req, row0, None, 1, split, waves))
+            lists.append((req, row0, None, 1, split, waves, False))
         if large:
-            req, row0, row1 = ops.attention_tiles(q_lens, group, 2, large, pair=True)
             whole = -(-max(bound, 1) // 128) * 128
-            lists.append((req, row0, row1, 2, whole, 1))
+            wavefronts = sum(-(-q_lens[r] * group // 32) for r in large) * nkv
+            if page_size >= 16 and wavefronts >= ops.ATTENTION_GROUPED_FROM:
+                req, row0, _ = ops.attention_tiles(q_lens, group, 2, large, fill=ops.ATTENTION_GROUP)
+                lists.append((req, row0, None, 2, whole, 1, True))
+            else:
+                req, row0, row1 = ops.attention_tiles(q_lens, group, 2, large, pair=True)
+                lists.append((req, row0, row1, 2, whole, 1, False))
         # one upload for all the tile lists of the step
         flat = [x for req, row0, row1, *_ in lists for x in (req + row0 + (row1 or []))]
         dev = upload(flat, torch.int32, ctx.device) if flat else None
         launches, at = [], 0
-        for req, row0, row1, row_tiles, split, waves in lists:
+        for req, row0, row1, row_tiles, split, waves, grouped in lists:
             n = len(req)
             t_req, t_row0 = dev[at : at + n], dev[at + n : at + 2 * n]
             t_row1 = dev[at + 2 * n : at + 3 * n] if row1 is not None else None
             at += (3 if row1 is not None else 2) * n
             launches.append(AttentionLaunch(t_req, t_row0, t_row1, row_tiles, split, waves,
-                                            ops.AttentionScratch(ctx.device) if static else None))
+                                            ops.AttentionScratch(ctx.device) if static else None, grouped))
         plan = AttentionPlan(launches, bound)
         ctx.extras[key] = plan
     return plan
@@ -184,7 +192,7 @@ class PagedAttention(Mixer):
                 cache.keys, cache.values, nq, nkv, d, cache.page_size, write_cache=cache.writable,
             )
         if ops.attention_mfma_supports(q.dtype, d, cache.page_size):
-            plan = attention_plan(ctx, nq // nkv, nkv, d)
+            plan = attention_plan(ctx, nq // nkv, nkv, d, cache.page_size)
             attn = torch.empty((q.shape[0], nq * d), dtype=q.dtype, device=q.device)
             for launch in plan.launches:
                 ops.paged_attention_mfma(
@@ -192,6 +200,7 @@ class PagedAttention(Mixer):
                     launch.tile_req, launch.tile_row0, launch.row_tiles, nq, nkv, d, cache.page_size,
                     plan.max_kv_len, launch.split, window=self.window, scale=self.scale, waves=launch.waves,
                     out=attn, scratch=launch.scratch, tile_row1=launch.tile_row1, longest=ctx.max_kv_len,
+                    grouped=launch.grouped,
                 )
         else:
             # the true 32-bit path, and shapes the matrix-core kernel does not take
