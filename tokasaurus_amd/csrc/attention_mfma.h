@@ -364,7 +364,8 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
     constexpr int NKR = (NK + GROUP_WAVES - 1) / GROUP_WAVES, NVR = (NV + GROUP_WAVES - 1) / GROUP_WAVES;
     int* ranges = (int*)wg_part;
     bf16x8_t* k_lds = (bf16x8_t*)(wg_part + 16);
-    bf16x4_t* v_lds = (bf16x4_t*)(k_lds + 2 * NK * 64);
+    // values: the two 16-key blocks of a fragment side by side, as the value product's operand wants them
+    bf16x8_t* v_lds = k_lds + 2 * NK * 64;  // [buffer][dt][lane]
     if (lane == 0) {
       ranges[2 * wave] = t.lo;
       ranges[2 * wave + 1] = t.hi;
@@ -426,7 +427,10 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
 #pragma unroll
       for (int i = 0; i < NVR; ++i) {
         const int f = i * GROUP_WAVES + wave;
-        if (f < NV) v_lds[(size_t)(buf * NV + f) * 64 + lane] = vreg[i];
+        if (f < NV) {
+          const int blk = f / DT, dt = f - blk * DT;
+          ((bf16x4_t*)(v_lds + (size_t)(buf * DT + dt) * 64 + lane))[blk] = vreg[i];
+        }
       }
     };
     StepPages pg = step_pages(a, table, g_begin, glo, ghi);
@@ -448,9 +452,9 @@ __device__ __forceinline__ void attention_item(const AttnArgs& a, const int tile
         for (int blk = 0; blk < 2; ++blk) {
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) cur.kv[blk][ks] = k_lds[(size_t)(buf * NK + blk * KS + ks) * 64 + lane];
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) cur.vv[dt].half[blk] = v_lds[(size_t)(buf * NV + blk * DT + dt) * 64 + lane];
         }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) cur.vv[dt].whole = v_lds[(size_t)(buf * DT + dt) * 64 + lane];
         compute_step(cur, kb);
       }
       __syncthreads();

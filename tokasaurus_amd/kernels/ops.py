@@ -353,8 +353,9 @@ def check_attention_shape(dtype: torch.dtype, nq: int, nkv: int, head_dim: int, 
 ATTENTION_GROUP = 4  # wavefronts (of two neighbouring row tiles each) in a workgroup of the grouped prompt kernel
 # Wavefronts (of two row tiles, over all kv heads) from which prompts take the grouped kernel: with
 # three and more a SIMD it is ahead of the kernel of paired tiles.  Measured on an MI355X, prefill
-# of one prompt, grouped against paired: 1B shape 2 048 tokens 5.85 / 5.70 ms, 4 096 tokens 10.2 /
-# 10.7 ms, 8 192 tokens 22.2 / 24.7 ms; 8B shape 4 096 tokens 51.6 / 54.3 ms, 8 192 tokens 114 / 128 ms.
+# of one prompt, grouped against paired: 1B shape 2 048 tokens 5.98 / 5.77 ms, 3 072 tokens 8.10 /
+# 8.54 ms, 4 096 tokens 9.8 / 10.7 ms, 8 192 tokens 20.3 / 24.7 ms; 8B shape 2 048 tokens 28.0 / 28.1
+# ms, 4 096 tokens 50.2 / 53.8 ms, 8 192 tokens 110 / 128 ms.
 ATTENTION_GROUPED_FROM = 3072
 
 
